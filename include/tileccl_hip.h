@@ -1,0 +1,239 @@
+/*
+ * tileccl_hip.h -- C ABI of libtileccl_hip.so (gfx950 / MI355X).
+ *
+ * The reference is pure Python + Triton: its host code reaches the GPU through Triton
+ * launches (`kernel[grid](...)`) and, for the runtime, through ctypes into libamdhip64
+ * (/root/reference/tileccl/backends/hip.py:67-186).  Each entry point below replaces
+ * one of those launch sites with a hand-written HIP kernel; the comment on each names
+ * the reference launch it stands in for.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t, or a negative
+ *     tccl_status; tccl_last_error_string() describes the last failure on the calling
+ *     thread.  Nothing throws, nothing touches Python.
+ *   - all pointers inside descriptors are DEVICE pointers valid for the duration of the
+ *     call's stream work; the library never owns tensor memory.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Launches
+ *     are asynchronous; no entry point synchronises the device.
+ *   - matrices are row-major; leading dimensions are in elements.
+ *   - not re-entrant across host threads for one device (same as the reference, which
+ *     keeps process-global context state: tileccl/__init__.py:228).
+ */
+#ifndef TILECCL_HIP_H
+#define TILECCL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCCL_ABI_VERSION 1
+#define TCCL_MAX_WORLD 8
+
+typedef enum tccl_status {
+  TCCL_OK = 0,
+  TCCL_ERR_INVALID = -1,     /* bad argument / descriptor */
+  TCCL_ERR_UNSUPPORTED = -2, /* layout, dtype or shape this build has no kernel for */
+  TCCL_ERR_NO_DEVICE = -3,
+  TCCL_ERR_TIMEOUT = -4      /* a bounded device-side wait expired (see tccl_read_fault) */
+} tccl_status;
+
+typedef enum tccl_dtype {
+  TCCL_F16 = 0,
+  TCCL_BF16 = 1,
+  TCCL_F32 = 2,
+  TCCL_F8E4M3 = 3 /* OCP e4m3fn, max 448: the fp8 format of gfx950 MFMA */
+} tccl_dtype;
+
+/* S0 bulk / S1 tile-by-tile / S2 TileGroup (reference README.md:66-84). */
+typedef enum tccl_variant {
+  TCCL_S0_BULK = 0,
+  TCCL_S1_TILE = 1,
+  TCCL_S2_TILEGROUP = 2
+} tccl_variant;
+
+/* Transfer directions carried out by one launch (bit mask).  PUSH: this rank's rows go
+ * to the peers (reference tileccl_v2/transport.py:18 CommMode.PUSH).  PULL: the peers'
+ * rows are read into this rank's slice (CommMode.PULL).  On one GPU, PUSH|PULL runs both
+ * halves of a two-rank exchange through the same HBM. */
+#define TCCL_DIR_PUSH 1
+#define TCCL_DIR_PULL 2
+
+typedef struct tccl_device_info {
+  int32_t compute_units;   /* CUs (256 on MI355X) */
+  int32_t clock_khz;       /* engine clock */
+  int32_t lds_bytes;       /* LDS per workgroup limit */
+  int32_t wavefront;       /* 64 */
+  int32_t xcds;            /* accelerator dies sharing one L2 each (8 on MI355X) */
+  int32_t reserved[3];
+  char arch[64];           /* "gfx950..." */
+} tccl_device_info;
+
+/* ---- one GEMM: C[M,N] = alpha * A[M,K] @ B[K,N], fp32 accumulate ------------------
+ * Stands in for gemm_kernel (tileccl/kernels/gemm.py:53-167) and the GEMM bodies of the
+ * patterns (patterns/bulk_sync.py:162-238, wg_specialized.py:263-310).
+ * A must be k-contiguous (lda = row stride), B n-contiguous (ldb = row stride).
+ * Plan tiles are block_m x block_n; tile ids follow the group_m swizzle of the
+ * reference GEMM (kernels/gemm.py:118-123) so that they index group_table / locks. */
+typedef struct tccl_gemm_desc {
+  const void* A;
+  const void* B;
+  void* C;
+  int32_t M, N, K;
+  int64_t lda, ldb, ldc;
+  int32_t in_dtype;  /* tccl_dtype of A and B: F16, BF16 or F8E4M3 */
+  int32_t out_dtype; /* tccl_dtype of C: F16, BF16 or F32 */
+  float alpha;       /* applied to the fp32 accumulator (fp8: scale_a * scale_b) */
+  int32_t block_m, block_n, group_m; /* plan tile and swizzle band: 128/128/8 or 256/128/8 */
+  int32_t num_wgs;   /* GEMM workgroups; 0 = library default for the device */
+  int32_t reserved[3];
+} tccl_gemm_desc;
+
+/* ---- per-launch synchronisation words ------------------------------------------------
+ * Stands in for the lock tensor of WGSpecializedPattern (wg_specialized.py:104-124) and
+ * for TileGroupSignalState (tileccl_v2/signal.py:14-40).
+ *   locks      int32[total_tiles]   S1: tile_signal / tile_wait (sync/primitives.py:357-414)
+ *   group_table int32[total_tiles]  S2: swizzled tile id -> group id (tile_group.py:214-241)
+ *   counter    int32[n_groups]      S2: tile_signal_add / tile_wait_ge (tileccl_v2/ipc.py:231-254)
+ *   barrier    int32[n_groups]      S2: finished communication tasks per group
+ *   trace_*    optional device-clock stamps (signal.py:18-24); NULL to skip
+ * locks, counter and barrier live in the symmetric heap, so a peer's copy sits at the
+ * same offset in the peer's slice.  The host zeroes them before a launch
+ * (TileGroupSignalState.reset, signal.py:32-40); `epoch` lets repeated launches reuse
+ * unreset counters: a group is ready when counter[g] >= epoch * tile_counts[g]. */
+typedef struct tccl_sync_desc {
+  int32_t* locks;
+  const int32_t* group_table;
+  int32_t* counter;
+  int32_t* barrier;
+  int32_t n_groups;
+  int32_t epoch; /* >= 1 */
+  const int32_t* row_starts; /* int32[n_groups], rows relative to the GEMM's C */
+  const int32_t* row_ends;   /* clamped to M */
+  const int32_t* tile_counts;
+  int32_t* trace_comm_counter;  /* int32[n_groups] or NULL */
+  int64_t* trace_start_clock;   /* int64[1] or NULL */
+  int64_t* trace_ready_clock;   /* int64[n_groups] or NULL */
+  int64_t* trace_done_clock;    /* int64[n_groups] or NULL */
+  int64_t* fault;               /* int64[1] or NULL: set non-zero if a bounded wait expired */
+  int64_t spin_limit_ns;        /* bound of every device-side wait; 0 = library default (2 s) */
+} tccl_sync_desc;
+
+/* ---- symmetric heap view -------------------------------------------------------------
+ * heap_bases is the int64[world_size] device array of slice base addresses
+ * (tileccl_v2/heap.py:143-145, memory/symmetric_heap.py:929-938); rank / world_size as
+ * in the reference context.  translate(ptr, to) = heap_bases[to] + (ptr - heap_bases[rank])
+ * (memory/translation.py:39-99). */
+typedef struct tccl_heap_view {
+  const int64_t* heap_bases;
+  int32_t rank;
+  int32_t world_size;
+} tccl_heap_view;
+
+/* ---- all-scatter placement (tileccl.ops.gemm_allscatter) ------------------------------
+ * The four integers of PatternExecutionSpec (patterns/contracts.py:206-215) consumed by
+ * scatter_tile_to_peer (patterns/_helpers.py:145-157): columns
+ * [src_col_offset, src_col_offset+cols) of the local C go to every peer's C at
+ * row*dst_ld + dst_col_offset + (col - src_col_offset). */
+typedef struct tccl_scatter_desc {
+  int32_t src_col_offset;
+  int32_t cols;
+  int32_t dst_ld;
+  int32_t dst_col_offset;
+} tccl_scatter_desc;
+
+/* ---- transport knobs (tileccl_v2/transport.py:23-53, wg.py:10-51) --------------------- */
+typedef struct tccl_transport_desc {
+  int32_t directions;   /* TCCL_DIR_* mask */
+  int32_t copy_elems;   /* elements per copy task */
+  int32_t reduce_elems; /* elements per reduce task (0: use copy_elems) */
+  int32_t num_comm_wgs; /* communication workgroups of a fused launch; 0 = default */
+} tccl_transport_desc;
+
+/* ---- runtime -------------------------------------------------------------------------*/
+int tccl_abi_version(void);
+const char* tccl_last_error_string(void);
+/* backends/hip.py:458-490 get_device_properties (compute_units et al.). */
+int tccl_device_query(int device, tccl_device_info* out);
+/* Pure host helper: swizzled tile id -> (tile_m, tile_n); same code the kernels run
+ * (kernels/gemm.py:118-123).  Exposed so CPU tests can pin the device-side index math. */
+int tccl_tile_coords(int32_t tile_id, int32_t tile_rows, int32_t tile_cols, int32_t group_m,
+                     int32_t* tile_m, int32_t* tile_n);
+/* Pure host helper: launch slot -> swizzled tile id after the XCD-aware remap (each XCD
+ * takes `span` consecutive ids out of every block of xcds*span). */
+int tccl_tile_for_slot(int32_t slot, int32_t total_tiles, int32_t xcds, int32_t span, int32_t* tile_id);
+
+/* ---- symmetric heap: one hipMalloc arena cut into world_size slices -------------------
+ * Replaces one torch.empty per rank + IPC/peer mapping (tileccl_v2/heap.py:137,225-264;
+ * memory/symmetric_heap.py:239-343).  bases_out: host int64[world_size]. */
+int tccl_heap_create(size_t slice_bytes, int world_size, void** arena_out, int64_t* bases_out);
+int tccl_heap_destroy(void* arena);
+
+/* ---- small device utilities ---------------------------------------------------------- */
+/* Fill kernel (never hipMemsetAsync): signal reset, signal.py:32-40. */
+int tccl_fill_i32(int32_t* words, int64_t n, int32_t value, void* stream);
+/* Single-word primitives, one launch each, for tests of the device semantics
+ * (sync/primitives.py:357-500, tileccl_v2/ipc.py:137-254).  result: device int32[1]. */
+int tccl_prim_signal(int32_t* locks, int32_t index, void* stream);
+int tccl_prim_signal_add(int32_t* words, int32_t index, int32_t value, int32_t* result, void* stream);
+int tccl_prim_try_wait(int32_t* locks, int32_t index, int32_t max_spins, int32_t consume,
+                       int32_t* result, void* stream);
+int tccl_prim_wait_ge(int32_t* words, int32_t index, int32_t threshold, int64_t spin_limit_ns,
+                      int32_t* result, void* stream);
+
+/* ---- GEMM alone ------------------------------------------------------------------------ */
+int tccl_gemm(const tccl_gemm_desc* gemm, void* stream);
+
+/* ---- communication phases alone (the second kernel of S0) ------------------------------
+ * tccl_scatter_cols: BulkSyncPattern._scatter_kernel (patterns/bulk_sync.py:242-299).
+ * elem_bytes: size of one element of C. */
+int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes,
+                      const tccl_scatter_desc* scatter, const tccl_heap_view* heap, void* stream);
+/* tccl_exchange_rows: the row-block exchange of GEMM-output AllGather
+ * (tile_allgather layout [block_rank0 | block_rank1 | ...], primitives/collectives.py:613-663).
+ * `out` is this rank's gathered output (world*rows_per_rank x N, leading dim ld) in its
+ * slice; rank r's block occupies rows [r*rows_per_rank, (r+1)*rows_per_rank). */
+int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, int32_t elem_bytes,
+                       const tccl_heap_view* heap, const tccl_transport_desc* transport, void* stream);
+/* tccl_reduce_rows: pull-reduce of tile_reduce_scatter (collectives.py:730-783) over row
+ * shards with fp32 accumulation: out[r - row_lo] = cast(sum_p partial_p[r]) for
+ * r in [row_lo, row_hi), where partial_p is `partial` translated into slice p, summed
+ * local first, then peers in ascending rank.  If `emulate_peer` is non-zero the same
+ * reduction is also carried out for every other rank's shard into that rank's `out`. */
+int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_partial, void* out,
+                     int32_t out_dtype, int64_t ld_out, int32_t M, int32_t N,
+                     const tccl_heap_view* heap, const tccl_transport_desc* transport,
+                     int32_t emulate_peer, void* stream);
+
+/* ---- fused operations --------------------------------------------------------------------
+ * variant S0: GEMM kernel, then the communication kernel, stream-ordered.
+ * variant S1: one launch; GEMM workgroups signal locks[tile]; communication workgroups
+ *             wait per tile (WGSpecializedPattern, wg_specialized.py:212-352).
+ * variant S2: one launch; GEMM workgroups add to counter[group_table[tile]];
+ *             communication workgroups wait per TileGroup and move copy_elems-sized
+ *             tasks (reference README.md:66-84; contract in tileccl_v2/*.py). */
+
+/* tileccl.ops.gemm_allscatter (ops.py:810-888): C = A@B locally, then the rank's column
+ * block is stored into every peer's C. */
+int tccl_gemm_allscatter(const tccl_gemm_desc* gemm, const tccl_scatter_desc* scatter,
+                         const tccl_heap_view* heap, const tccl_sync_desc* sync,
+                         const tccl_transport_desc* transport, int32_t variant, void* stream);
+
+/* GEMM-output AllGather (Gate 1).  gemm->C must point at row rank*M of `out`. */
+int tccl_gemm_allgather(const tccl_gemm_desc* gemm, void* out, int64_t ld_out,
+                        const tccl_heap_view* heap, const tccl_sync_desc* sync,
+                        const tccl_transport_desc* transport, int32_t variant, void* stream);
+
+/* GEMM to ReduceScatter (Gate 2).  gemm->C is the rank's partial (M x N, dtype
+ * gemm->out_dtype) in its slice; `out` receives the rank's M/world_size row shard. */
+int tccl_gemm_reducescatter(const tccl_gemm_desc* gemm, void* out, int32_t out_dtype, int64_t ld_out,
+                            const tccl_heap_view* heap, const tccl_sync_desc* sync,
+                            const tccl_transport_desc* transport, int32_t emulate_peer,
+                            int32_t variant, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TILECCL_HIP_H */

@@ -1,0 +1,198 @@
+"""Marshalling between torch tensors and the C ABI descriptors.
+
+Everything here is host bookkeeping: it validates what the kernels assume (contiguity,
+dtypes, device) and hands raw device pointers down.  The launches go to torch's current
+stream, like the reference's Triton launches do.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+
+import torch
+
+from tileccl_amd import _lib
+
+_DTYPE_CODES = {
+    torch.float16: _lib.F16,
+    torch.bfloat16: _lib.BF16,
+    torch.float32: _lib.F32,
+}
+if hasattr(torch, "float8_e4m3fn"):
+    _DTYPE_CODES[torch.float8_e4m3fn] = _lib.F8E4M3
+
+VARIANTS = {"s0": _lib.S0_BULK, "s1": _lib.S1_TILE, "s2": _lib.S2_TILEGROUP}
+DEFAULT_SPIN_LIMIT_NS = 2_000_000_000
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype {dtype} is not supported by the HIP kernels") from None
+
+
+def stream_ptr() -> int:
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else int(t.data_ptr())
+
+
+def _row_major(t: torch.Tensor, name: str) -> int:
+    """Leading dimension of a 2-D tensor whose rows are contiguous."""
+    if t.ndim != 2:
+        raise ValueError(f"{name} must be 2-D, got {t.ndim}-D")
+    if t.shape[1] > 1 and t.stride(1) != 1:
+        raise ValueError(
+            f"{name} must have contiguous rows (stride(1) == 1), got strides {tuple(t.stride())}; "
+            "call .contiguous() first"
+        )
+    return int(t.stride(0)) if t.shape[0] > 1 else int(t.shape[1])
+
+
+def gemm_desc(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    C_out: torch.Tensor,
+    *,
+    block_m: int = 128,
+    block_n: int = 128,
+    group_m: int = 8,
+    alpha: float = 1.0,
+    num_wgs: int = 0,
+) -> _lib.GemmDesc:
+    if not (A.is_cuda and B.is_cuda and C_out.is_cuda):
+        raise ValueError("GEMM operands must be device tensors")
+    if A.dtype != B.dtype:
+        raise ValueError(f"A and B must share a dtype, got {A.dtype} and {B.dtype}")
+    M, K = A.shape
+    K2, N = B.shape
+    if K2 != K:
+        raise ValueError(f"B.shape[0] must equal A.shape[1]: got {K2} vs {K}")
+    if tuple(C_out.shape) != (M, N):
+        raise ValueError(f"C shape mismatch: expected ({M}, {N}), got {tuple(C_out.shape)}")
+    d = _lib.GemmDesc()
+    d.A, d.B, d.C = ptr(A), ptr(B), ptr(C_out)
+    d.M, d.N, d.K = int(M), int(N), int(K)
+    d.lda, d.ldb, d.ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C_out, "C")
+    d.in_dtype, d.out_dtype = dtype_code(A.dtype), dtype_code(C_out.dtype)
+    d.alpha = float(alpha)
+    d.block_m, d.block_n, d.group_m = int(block_m), int(block_n), int(group_m)
+    d.num_wgs = int(num_wgs)
+    return d
+
+
+def heap_view(heap_bases: torch.Tensor, rank: int, world_size: int) -> _lib.HeapView:
+    v = _lib.HeapView()
+    v.heap_bases = ptr(heap_bases)
+    v.rank, v.world_size = int(rank), int(world_size)
+    return v
+
+
+def transport_desc(directions: int, copy_elems: int, reduce_elems: int | None, num_comm_wgs: int) -> _lib.TransportDesc:
+    t = _lib.TransportDesc()
+    t.directions = int(directions)
+    t.copy_elems = int(copy_elems)
+    t.reduce_elems = int(reduce_elems or 0)
+    t.num_comm_wgs = int(num_comm_wgs)
+    return t
+
+
+@dataclass
+class DevicePlan:
+    """Device-resident copy of a ``TileGroupPlan``'s vectors (uploaded once per plan)."""
+
+    n_groups: int
+    group_table: torch.Tensor
+    row_starts: torch.Tensor
+    row_ends: torch.Tensor
+    tile_counts: torch.Tensor
+
+    @classmethod
+    def upload(cls, plan, device: str = "cuda:0") -> "DevicePlan":
+        def dev(values) -> torch.Tensor:
+            return torch.tensor(list(values), dtype=torch.int32, device=device)
+
+        return cls(
+            n_groups=plan.n_groups,
+            group_table=plan.group_table.to(device=device, dtype=torch.int32).contiguous(),
+            row_starts=dev(plan.row_starts()),
+            row_ends=dev(plan.row_ends()),
+            tile_counts=dev(plan.tile_counts()),
+        )
+
+
+@dataclass
+class SyncWords:
+    """Signal words of one fused operation plus the launch epoch.
+
+    Counters grow monotonically: launch ``e`` (1-based) treats group ``g`` as ready at
+    ``counter[g] >= e * tile_counts[g]``, so repeated launches need no reset kernel.
+    ``reset()`` zeroes the words and restarts the epoch, which is also what happens
+    automatically before the 32-bit counters could overflow.
+    """
+
+    locks: torch.Tensor | None = None
+    counter: torch.Tensor | None = None
+    barrier: torch.Tensor | None = None
+    plan: DevicePlan | None = None
+    host_plan: object | None = None  # the TileGroupPlan `plan` was uploaded from
+    trace_comm_counter: torch.Tensor | None = None
+    trace_start_clock: torch.Tensor | None = None
+    trace_ready_clock: torch.Tensor | None = None
+    trace_done_clock: torch.Tensor | None = None
+    fault: torch.Tensor = field(default_factory=lambda: torch.zeros(1, dtype=torch.int64, device="cuda:0"))
+    epoch: int = 0
+    spin_limit_ns: int = DEFAULT_SPIN_LIMIT_NS
+    max_tasks_per_tile: int = 1 << 16
+
+    def reset(self) -> None:
+        for t in (self.locks, self.counter, self.barrier, self.trace_comm_counter, self.trace_start_clock,
+                  self.trace_ready_clock, self.trace_done_clock, self.fault):
+            if t is not None:
+                t.zero_()
+        self.epoch = 0
+
+    def next_epoch(self) -> int:
+        if self.epoch >= (1 << 30) // self.max_tasks_per_tile:
+            torch.cuda.current_stream().synchronize()
+            self.reset()
+        self.epoch += 1
+        return self.epoch
+
+    def desc(self) -> _lib.SyncDesc:
+        s = _lib.SyncDesc()
+        s.locks = ptr(self.locks)
+        s.counter = ptr(self.counter)
+        s.barrier = ptr(self.barrier)
+        if self.plan is not None:
+            s.group_table = ptr(self.plan.group_table)
+            s.row_starts = ptr(self.plan.row_starts)
+            s.row_ends = ptr(self.plan.row_ends)
+            s.tile_counts = ptr(self.plan.tile_counts)
+            s.n_groups = self.plan.n_groups
+        s.epoch = max(self.epoch, 1)
+        s.trace_comm_counter = ptr(self.trace_comm_counter)
+        s.trace_start_clock = ptr(self.trace_start_clock)
+        s.trace_ready_clock = ptr(self.trace_ready_clock)
+        s.trace_done_clock = ptr(self.trace_done_clock)
+        s.fault = ptr(self.fault)
+        s.spin_limit_ns = int(self.spin_limit_ns)
+        return s
+
+    def raise_if_faulted(self) -> None:
+        """Synchronises the stream; raises if a device-side wait ran into its deadline."""
+        torch.cuda.current_stream().synchronize()
+        if int(self.fault.item()) != 0:
+            self.fault.zero_()
+            raise RuntimeError(
+                "a communication workgroup gave up waiting for a tile/TileGroup signal "
+                f"(spin limit {self.spin_limit_ns} ns); the output of this launch is incomplete"
+            )
+
+
+def byref(x):
+    return C.byref(x) if x is not None else None

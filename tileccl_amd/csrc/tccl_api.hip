@@ -1,0 +1,615 @@
+// Host side of libtileccl_hip.so: argument checks, launch geometry, and the extern "C"
+// entry points declared in include/tileccl_hip.h.  No Python, no torch types.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/tileccl_hip.h"
+#include "tccl_comm.h"
+#include "tccl_gemm.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail((int)e, "HIP error in %s: %s (%d)", what, hipGetErrorString(e), (int)e);
+}
+
+#define TCCL_HIP(call)                                  \
+  do {                                                  \
+    hipError_t e_ = (call);                             \
+    if (e_ != hipSuccess) return hip_fail(e_, #call);   \
+  } while (0)
+
+struct DeviceCache {
+  bool valid = false;
+  int device = -1;
+  tccl_device_info info;
+};
+DeviceCache g_dev;
+
+int query_device(int device, tccl_device_info* out) {
+  if (device < 0) TCCL_HIP(hipGetDevice(&device));
+  if (!g_dev.valid || g_dev.device != device) {
+    hipDeviceProp_t p;
+    TCCL_HIP(hipGetDeviceProperties(&p, device));
+    tccl_device_info i;
+    memset(&i, 0, sizeof i);
+    i.compute_units = p.multiProcessorCount;
+    i.clock_khz = p.clockRate;
+    i.lds_bytes = (int)p.sharedMemPerBlock;
+    i.wavefront = p.warpSize;
+    strncpy(i.arch, p.gcnArchName, sizeof(i.arch) - 1);
+    // MI300/MI350 class parts expose 8 accelerator dies; each owns compute_units / 8 CUs
+    // and one L2.  Smaller parts are treated as one die.
+    i.xcds = (i.compute_units >= 64 && i.compute_units % 8 == 0) ? 8 : 1;
+    g_dev.info = i;
+    g_dev.device = device;
+    g_dev.valid = true;
+  }
+  *out = g_dev.info;
+  return 0;
+}
+
+size_t dtype_size(int dt) {
+  switch (dt) {
+    case TCCL_F16:
+    case TCCL_BF16: return 2;
+    case TCCL_F32: return 4;
+    case TCCL_F8E4M3: return 1;
+    default: return 0;
+  }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// ------------------------------------------------------------------------------------------
+// Kernels
+// ------------------------------------------------------------------------------------------
+// One launch holds both roles: workgroups [0, num_compute) run the GEMM, the rest move
+// data.  Three waves per SIMD (two GEMM workgroups plus one communication workgroup per
+// CU) bounds the register budget.
+template <typename InT, typename OutT>
+__global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::SignalArgs s, tccl::CommArgs c,
+                                                       int num_compute, int64_t* trace_start) {
+  __shared__ __attribute__((aligned(16))) char smem[tccl::kLdsBytes];
+  if ((int)blockIdx.x < num_compute) {
+    if (trace_start && blockIdx.x == 0 && threadIdx.x == 0) *trace_start = tccl::now_ticks();
+    tccl::GemmRole<InT, OutT>(g, smem).run(s, (int)blockIdx.x, num_compute);
+  } else {
+    tccl::comm_role(c, (int)blockIdx.x - num_compute, (int)gridDim.x - num_compute, (int*)smem);
+  }
+}
+
+__global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
+  __shared__ int word[4];
+  tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
+}
+
+__global__ void fill_kernel(int32_t* w, int64_t n, int32_t v) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) w[i] = v;
+}
+
+__global__ void prim_signal_kernel(int32_t* locks, int i) { tccl::tile_signal(locks, i); }
+__global__ void prim_signal_add_kernel(int32_t* w, int i, int v, int32_t* res) { *res = tccl::tile_signal_add(w, i, v); }
+__global__ void prim_try_wait_kernel(int32_t* locks, int i, int spins, int consume, int32_t* res) {
+  *res = tccl::tile_try_wait(locks, i, spins, consume != 0) ? 1 : 0;
+}
+__global__ void prim_wait_ge_kernel(int32_t* w, int i, int thr, int64_t ticks, int32_t* res) {
+  *res = tccl::tile_wait_ge(w, i, thr, tccl::now_ticks() + ticks) ? 1 : 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Argument translation
+// ------------------------------------------------------------------------------------------
+constexpr int64_t kDefaultSpinNs = 2000000000ll;
+
+int check_gemm(const tccl_gemm_desc* d) {
+  if (!d) return fail(TCCL_ERR_INVALID, "gemm descriptor is NULL");
+  if (!d->A || !d->B || !d->C) return fail(TCCL_ERR_INVALID, "gemm: A, B and C must be non-NULL");
+  if (d->M <= 0 || d->N <= 0 || d->K <= 0) return fail(TCCL_ERR_INVALID, "gemm: M, N, K must be positive (got %d, %d, %d)", d->M, d->N, d->K);
+  if (d->block_m <= 0 || d->block_n <= 0 || d->group_m <= 0) return fail(TCCL_ERR_INVALID, "gemm: block_m, block_n, group_m must be positive");
+  if (d->block_m % tccl::kTile || d->block_n % tccl::kTile)
+    return fail(TCCL_ERR_UNSUPPORTED, "gemm: plan tile %dx%d must be a multiple of 128x128", d->block_m, d->block_n);
+  const size_t isz = dtype_size(d->in_dtype), osz = dtype_size(d->out_dtype);
+  if (!isz || !osz) return fail(TCCL_ERR_INVALID, "gemm: unknown dtype");
+  if (d->in_dtype == TCCL_F32) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp32 inputs have no MFMA kernel here");
+  if (d->out_dtype == TCCL_F8E4M3) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 output is not supported");
+  const int in_vec = (int)(16 / isz), out_vec = (int)(16 / osz);
+  if (d->K % in_vec) return fail(TCCL_ERR_UNSUPPORTED, "gemm: K=%d must be a multiple of %d", d->K, in_vec);
+  if (d->N % 8) return fail(TCCL_ERR_UNSUPPORTED, "gemm: N=%d must be a multiple of 8", d->N);
+  if (d->lda < d->K || d->ldb < d->N || d->ldc < d->N) return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
+  if (d->lda % in_vec || d->ldb % in_vec || d->ldc % out_vec || !aligned16(d->A) || !aligned16(d->B) || !aligned16(d->C))
+    return fail(TCCL_ERR_UNSUPPORTED, "gemm: A, B, C rows must start on 16-byte boundaries");
+  return 0;
+}
+
+int gemm_span(int per_band, int group_m, int tile_cols, int xcds) {
+  // Tile ids an XCD takes from each block: whole columns of a band, as close to
+  // per_band / xcds as divides evenly.
+  if (xcds <= 1) return 1;
+  int cols = tile_cols / xcds;
+  if (cols < 1) cols = 1;
+  (void)per_band;
+  return cols * group_m;
+}
+
+int build_gemm_args(const tccl_gemm_desc* d, const tccl_device_info& dev, tccl::GemmArgs* g) {
+  g->A = d->A;
+  g->B = d->B;
+  g->C = d->C;
+  g->M = d->M;
+  g->N = d->N;
+  g->K = d->K;
+  g->lda = d->lda;
+  g->ldb = d->ldb;
+  g->ldc = d->ldc;
+  g->alpha = d->alpha;
+  g->block_m = d->block_m;
+  g->block_n = d->block_n;
+  g->group_m = d->group_m;
+  g->tile_rows = (d->M + d->block_m - 1) / d->block_m;
+  g->tile_cols = (d->N + d->block_n - 1) / d->block_n;
+  g->xcds = dev.xcds;
+  g->span = gemm_span(d->group_m * g->tile_cols, d->group_m, g->tile_cols, dev.xcds);
+  return 0;
+}
+
+int default_gemm_wgs(const tccl_gemm_desc* d, const tccl_device_info& dev, int total_tiles) {
+  int n = d->num_wgs > 0 ? d->num_wgs : 2 * dev.compute_units;
+  if (n > total_tiles) n = total_tiles;
+  return n < 1 ? 1 : n;
+}
+
+void fill_comm_common(tccl::CommArgs* c, const tccl::GemmArgs& g, int esize, const tccl_heap_view* heap,
+                      const tccl_sync_desc* sync, const tccl_transport_desc* tr) {
+  memset(c, 0, sizeof *c);
+  c->heap_bases = heap->heap_bases;
+  c->rank = heap->rank;
+  c->world = heap->world_size;
+  c->C = (char*)g.C;
+  c->ldc_bytes = g.ldc * esize;
+  c->M = g.M;
+  c->N = g.N;
+  c->esize = esize;
+  c->block_m = g.block_m;
+  c->block_n = g.block_n;
+  c->group_m = g.group_m;
+  c->tile_rows = g.tile_rows;
+  c->tile_cols = g.tile_cols;
+  c->xcds = g.xcds;
+  c->span = g.span;
+  c->directions = tr ? tr->directions : TCCL_DIR_PUSH;
+  c->n_groups = 1;
+  c->epoch = 1;
+  c->spin_ticks = kDefaultSpinNs / 10;
+  if (sync) {
+    c->locks = sync->locks;
+    c->counter = sync->counter;
+    c->barrier = sync->barrier;
+    c->row_starts = sync->row_starts;
+    c->row_ends = sync->row_ends;
+    c->tile_counts = sync->tile_counts;
+    if (sync->row_starts && sync->n_groups > 0) c->n_groups = sync->n_groups;
+    c->epoch = sync->epoch > 0 ? sync->epoch : 1;
+    c->trace_comm_counter = sync->trace_comm_counter;
+    c->trace_ready_clock = sync->trace_ready_clock;
+    c->trace_done_clock = sync->trace_done_clock;
+    c->fault = sync->fault;
+    if (sync->spin_limit_ns > 0) c->spin_ticks = sync->spin_limit_ns / 10 + 1;
+  }
+}
+
+int check_heap(const tccl_heap_view* h) {
+  if (!h || !h->heap_bases) return fail(TCCL_ERR_INVALID, "heap view / heap_bases is NULL");
+  if (h->world_size < 1 || h->world_size > TCCL_MAX_WORLD) return fail(TCCL_ERR_INVALID, "world_size=%d outside [1, %d]", h->world_size, TCCL_MAX_WORLD);
+  if (h->rank < 0 || h->rank >= h->world_size) return fail(TCCL_ERR_INVALID, "rank=%d out of range for world_size=%d", h->rank, h->world_size);
+  return 0;
+}
+
+int set_task_units(tccl::CommArgs* c, const tccl_transport_desc* tr, bool reduce) {
+  const int unit_elems = reduce ? 8 : 16 / c->esize;
+  int elems = tr ? (reduce && tr->reduce_elems > 0 ? tr->reduce_elems : tr->copy_elems) : 0;
+  if (elems <= 0) elems = 16384;
+  if (elems % unit_elems) return fail(TCCL_ERR_UNSUPPORTED, "task size %d elements is not a multiple of %d", elems, unit_elems);
+  c->copy_units = c->reduce_units = elems / unit_elems;
+  return 0;
+}
+
+int check_sync(const tccl_sync_desc* s, int variant) {
+  if (variant == TCCL_S0_BULK) return 0;
+  if (!s) return fail(TCCL_ERR_INVALID, "variant S%d needs a sync descriptor", variant);
+  if (variant == TCCL_S1_TILE && !s->locks) return fail(TCCL_ERR_INVALID, "S1 needs locks");
+  if (variant == TCCL_S2_TILEGROUP) {
+    if (!s->counter || !s->group_table || !s->row_starts || !s->row_ends || !s->tile_counts || s->n_groups <= 0)
+      return fail(TCCL_ERR_INVALID, "S2 needs counter, group_table, row_starts, row_ends, tile_counts and n_groups > 0");
+    if (s->epoch < 1) return fail(TCCL_ERR_INVALID, "S2 epoch must be >= 1");
+  }
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Launchers
+// ------------------------------------------------------------------------------------------
+template <typename InT, typename OutT>
+int launch_fused_t(const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c, int compute, int comm,
+                   int64_t* trace_start, hipStream_t stream) {
+  hipLaunchKernelGGL((fused_kernel<InT, OutT>), dim3(compute + comm), dim3(tccl::kThreads), 0, stream, g, s, c, compute,
+                     trace_start);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c,
+                 int compute, int comm, int64_t* trace_start, hipStream_t stream) {
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_fused_t<_Float16, _Float16>(g, s, c, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused_t<_Float16, float>(g, s, c, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused_t<__bf16, __bf16>(g, s, c, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused_t<__bf16, float>(g, s, c, compute, comm, trace_start, stream);
+  return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
+}
+
+int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
+  if (wgs < 1) wgs = 1;
+  hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int bulk_comm_wgs(const tccl_device_info& dev) { return dev.compute_units * 4; }
+
+// GEMM (+ optional communication role) for one of the three operations.
+int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc* sync, const tccl_transport_desc* tr,
+                int variant, const tccl_device_info& dev, const tccl::GemmArgs& g, hipStream_t stream) {
+  const int total_tiles = g.tile_rows * g.tile_cols;
+  const int compute = default_gemm_wgs(d, dev, total_tiles);
+  tccl::SignalArgs s;
+  memset(&s, 0, sizeof s);
+  int64_t* trace_start = sync ? sync->trace_start_clock : nullptr;
+  if (variant == TCCL_S0_BULK) {
+    tccl::CommArgs none;
+    memset(&none, 0, sizeof none);
+    int rc = launch_fused(d->in_dtype, d->out_dtype, g, s, none, compute, 0, trace_start, stream);
+    if (rc) return rc;
+    c.granularity = tccl::kBulk;
+    if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
+    return launch_comm(c, bulk_comm_wgs(dev), stream);
+  }
+  int comm = tr && tr->num_comm_wgs > 0 ? tr->num_comm_wgs : dev.compute_units;
+  if (variant == TCCL_S1_TILE) {
+    s.mode = tccl::kSignalTile;
+    s.locks = sync->locks;
+    c.granularity = tccl::kPerTile;
+  } else {
+    s.mode = tccl::kSignalGroup;
+    s.counter = sync->counter;
+    s.group_table = sync->group_table;
+    c.granularity = tccl::kPerGroup;
+  }
+  return launch_fused(d->in_dtype, d->out_dtype, g, s, c, compute, comm, trace_start, stream);
+}
+
+}  // namespace
+
+// ============================================================================================
+// extern "C"
+// ============================================================================================
+extern "C" {
+
+int tccl_abi_version(void) { return TCCL_ABI_VERSION; }
+
+const char* tccl_last_error_string(void) { return g_error; }
+
+int tccl_device_query(int device, tccl_device_info* out) {
+  if (!out) return fail(TCCL_ERR_INVALID, "out is NULL");
+  return query_device(device, out);
+}
+
+int tccl_tile_coords(int32_t tile_id, int32_t tile_rows, int32_t tile_cols, int32_t group_m, int32_t* tile_m, int32_t* tile_n) {
+  if (tile_rows <= 0 || tile_cols <= 0 || group_m <= 0 || tile_id < 0 || tile_id >= tile_rows * tile_cols || !tile_m || !tile_n)
+    return fail(TCCL_ERR_INVALID, "tile_coords: bad arguments");
+  const tccl::TileCoord c = tccl::tile_coords(tile_id, tile_rows, tile_cols, group_m);
+  *tile_m = c.m;
+  *tile_n = c.n;
+  return 0;
+}
+
+int tccl_tile_for_slot(int32_t slot, int32_t total_tiles, int32_t xcds, int32_t span, int32_t* tile_id) {
+  if (slot < 0 || slot >= total_tiles || xcds <= 0 || span <= 0 || !tile_id) return fail(TCCL_ERR_INVALID, "tile_for_slot: bad arguments");
+  *tile_id = tccl::tile_for_slot(slot, total_tiles, xcds, span);
+  return 0;
+}
+
+int tccl_heap_create(size_t slice_bytes, int world_size, void** arena_out, int64_t* bases_out) {
+  if (!arena_out || !bases_out) return fail(TCCL_ERR_INVALID, "heap_create: NULL output");
+  if (slice_bytes == 0) return fail(TCCL_ERR_INVALID, "heap_create: slice size must be positive");
+  if (world_size < 1 || world_size > TCCL_MAX_WORLD) return fail(TCCL_ERR_INVALID, "heap_create: world_size=%d outside [1, %d]", world_size, TCCL_MAX_WORLD);
+  // Slices start on 2 MiB boundaries so that symmetric offsets keep page alignment.
+  const size_t align = 2u << 20;
+  const size_t stride = (slice_bytes + align - 1) / align * align;
+  void* p = nullptr;
+  TCCL_HIP(hipMalloc(&p, stride * (size_t)world_size));
+  *arena_out = p;
+  for (int r = 0; r < world_size; ++r) bases_out[r] = (int64_t)(uintptr_t)p + (int64_t)(stride * (size_t)r);
+  return 0;
+}
+
+int tccl_heap_destroy(void* arena) {
+  if (!arena) return 0;
+  TCCL_HIP(hipFree(arena));
+  return 0;
+}
+
+int tccl_fill_i32(int32_t* words, int64_t n, int32_t value, void* stream) {
+  if (n <= 0) return 0;
+  if (!words) return fail(TCCL_ERR_INVALID, "fill: NULL pointer");
+  int blocks = (int)((n + 255) / 256);
+  if (blocks > 1024) blocks = 1024;
+  hipLaunchKernelGGL(fill_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, words, n, value);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_prim_signal(int32_t* locks, int32_t index, void* stream) {
+  if (!locks || index < 0) return fail(TCCL_ERR_INVALID, "prim_signal: bad arguments");
+  hipLaunchKernelGGL(prim_signal_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, locks, index);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_prim_signal_add(int32_t* words, int32_t index, int32_t value, int32_t* result, void* stream) {
+  if (!words || !result || index < 0) return fail(TCCL_ERR_INVALID, "prim_signal_add: bad arguments");
+  hipLaunchKernelGGL(prim_signal_add_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, words, index, value, result);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_prim_try_wait(int32_t* locks, int32_t index, int32_t max_spins, int32_t consume, int32_t* result, void* stream) {
+  if (!locks || !result || index < 0 || max_spins < 0) return fail(TCCL_ERR_INVALID, "prim_try_wait: bad arguments");
+  hipLaunchKernelGGL(prim_try_wait_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, locks, index, max_spins, consume, result);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_prim_wait_ge(int32_t* words, int32_t index, int32_t threshold, int64_t spin_limit_ns, int32_t* result, void* stream) {
+  if (!words || !result || index < 0) return fail(TCCL_ERR_INVALID, "prim_wait_ge: bad arguments");
+  if (spin_limit_ns <= 0 || spin_limit_ns > kDefaultSpinNs) spin_limit_ns = kDefaultSpinNs;
+  hipLaunchKernelGGL(prim_wait_ge_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, words, index, threshold, spin_limit_ns / 10 + 1, result);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_gemm(const tccl_gemm_desc* d, void* stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  build_gemm_args(d, dev, &g);
+  tccl::SignalArgs s;
+  memset(&s, 0, sizeof s);
+  tccl::CommArgs none;
+  memset(&none, 0, sizeof none);
+  return launch_fused(d->in_dtype, d->out_dtype, g, s, none, default_gemm_wgs(d, dev, g.tile_rows * g.tile_cols), 0, nullptr,
+                      (hipStream_t)stream);
+}
+
+static int check_scatter(const tccl_scatter_desc* sc, int M, int N, int esize, int64_t ldc, const void* C) {
+  if (!sc) return fail(TCCL_ERR_INVALID, "scatter descriptor is NULL");
+  if (sc->cols <= 0 || sc->src_col_offset < 0 || sc->dst_col_offset < 0 || sc->dst_ld <= 0)
+    return fail(TCCL_ERR_INVALID, "scatter: bad placement (src_col_offset=%d cols=%d dst_ld=%d dst_col_offset=%d)", sc->src_col_offset, sc->cols, sc->dst_ld, sc->dst_col_offset);
+  if (sc->src_col_offset + sc->cols > N) return fail(TCCL_ERR_INVALID, "scatter: source columns [%d, %d) exceed N=%d", sc->src_col_offset, sc->src_col_offset + sc->cols, N);
+  if (sc->dst_col_offset + sc->cols > sc->dst_ld) return fail(TCCL_ERR_INVALID, "scatter: destination columns exceed dst_ld");
+  const int v = 16 / esize;
+  if (sc->src_col_offset % v || sc->cols % v || sc->dst_col_offset % v || sc->dst_ld % v || ldc % v || !aligned16(C))
+    return fail(TCCL_ERR_UNSUPPORTED, "scatter: column offsets, widths and leading dimensions must be multiples of %d elements", v);
+  (void)M;
+  return 0;
+}
+
+int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes, const tccl_scatter_desc* sc,
+                      const tccl_heap_view* heap, void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  if (!C || M <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4)) return fail(TCCL_ERR_INVALID, "scatter_cols: bad arguments");
+  if (!sc) return fail(TCCL_ERR_INVALID, "scatter descriptor is NULL");
+  const int N = sc->src_col_offset + sc->cols;
+  if ((rc = check_scatter(sc, M, N, elem_bytes, ldc, C))) return rc;
+  if (heap->world_size == 1) return 0;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  memset(&g, 0, sizeof g);
+  g.C = (void*)C;
+  g.M = M;
+  g.N = N;
+  g.ldc = ldc;
+  g.block_m = g.block_n = 128;
+  g.group_m = 8;
+  g.tile_rows = (M + 127) / 128;
+  g.tile_cols = (N + 127) / 128;
+  g.xcds = 1;
+  g.span = 1;
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, elem_bytes, heap, nullptr, nullptr);
+  c.op = tccl::kOpAllScatter;
+  c.granularity = tccl::kBulk;
+  c.src_col_off = sc->src_col_offset;
+  c.cols = sc->cols;
+  c.dst_ld = sc->dst_ld;
+  c.dst_col_off = sc->dst_col_offset;
+  if ((rc = set_task_units(&c, nullptr, false))) return rc;
+  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+}
+
+int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, int32_t elem_bytes,
+                       const tccl_heap_view* heap, const tccl_transport_desc* tr, void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  if (!out || rows_per_rank <= 0 || N <= 0 || ld < N || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4))
+    return fail(TCCL_ERR_INVALID, "exchange_rows: bad arguments");
+  const int v = 16 / elem_bytes;
+  if (N % v || ld % v || !aligned16(out)) return fail(TCCL_ERR_UNSUPPORTED, "exchange_rows: rows must be multiples of 16 bytes");
+  if (heap->world_size == 1) return 0;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  memset(&g, 0, sizeof g);
+  g.C = (char*)out + (int64_t)heap->rank * rows_per_rank * ld * elem_bytes;
+  g.M = rows_per_rank;
+  g.N = N;
+  g.ldc = ld;
+  g.block_m = g.block_n = 128;
+  g.group_m = 8;
+  g.tile_rows = (rows_per_rank + 127) / 128;
+  g.tile_cols = (N + 127) / 128;
+  g.xcds = 1;
+  g.span = 1;
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, elem_bytes, heap, nullptr, tr);
+  c.op = tccl::kOpAllGather;
+  c.granularity = tccl::kBulk;
+  c.out = (char*)out;
+  c.ld_out_bytes = ld * elem_bytes;
+  if ((rc = set_task_units(&c, tr, false))) return rc;
+  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+}
+
+static int fill_reduce(tccl::CommArgs* c, const void* partial, int partial_dtype, void* out, int out_dtype, int64_t ld_out,
+                       int M, int N, int world, int emulate_peer) {
+  if (partial_dtype != TCCL_F16 && partial_dtype != TCCL_BF16 && partial_dtype != TCCL_F32)
+    return fail(TCCL_ERR_UNSUPPORTED, "reduce: partial dtype %d", partial_dtype);
+  if (out_dtype != TCCL_F16 && out_dtype != TCCL_BF16) return fail(TCCL_ERR_UNSUPPORTED, "reduce: output dtype must be fp16 or bf16");
+  if (partial_dtype != TCCL_F32 && partial_dtype != out_dtype && !(partial_dtype == TCCL_BF16 || partial_dtype == TCCL_F16))
+    return fail(TCCL_ERR_UNSUPPORTED, "reduce: dtype combination");
+  if (M % world) return fail(TCCL_ERR_INVALID, "reduce: M=%d must be divisible by world_size=%d", M, world);
+  if (N % 8 || ld_out % 8 || !aligned16(out) || !aligned16(partial)) return fail(TCCL_ERR_UNSUPPORTED, "reduce: rows must be multiples of 8 elements and 16-byte aligned");
+  c->op = tccl::kOpReduceScatter;
+  c->rs_out = (char*)out;
+  c->ld_rs_out_bytes = ld_out * 2;
+  c->partial_dtype = partial_dtype;
+  c->out_dtype = out_dtype;
+  c->emulate_peer = emulate_peer;
+  // Without a plan the kernel works shard by shard (one implicit group per owner).
+  if (!c->row_starts) c->n_groups = world;
+  return 0;
+}
+
+int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_partial, void* out, int32_t out_dtype,
+                     int64_t ld_out, int32_t M, int32_t N, const tccl_heap_view* heap, const tccl_transport_desc* tr,
+                     int32_t emulate_peer, void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  if (!partial || !out || M <= 0 || N <= 0 || ld_partial < N || ld_out < N) return fail(TCCL_ERR_INVALID, "reduce_rows: bad arguments");
+  const int esize = (int)dtype_size(partial_dtype);
+  if (!esize || ld_partial % (16 / esize)) return fail(TCCL_ERR_UNSUPPORTED, "reduce_rows: partial rows must be 16-byte multiples");
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  memset(&g, 0, sizeof g);
+  g.C = (void*)partial;
+  g.M = M;
+  g.N = N;
+  g.ldc = ld_partial;
+  g.block_m = g.block_n = 128;
+  g.group_m = 8;
+  g.tile_rows = (M + 127) / 128;
+  g.tile_cols = (N + 127) / 128;
+  g.xcds = 1;
+  g.span = 1;
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, esize, heap, nullptr, tr);
+  if ((rc = fill_reduce(&c, partial, partial_dtype, out, out_dtype, ld_out, M, N, heap->world_size, emulate_peer))) return rc;
+  c.granularity = tccl::kBulk;
+  if ((rc = set_task_units(&c, tr, true))) return rc;
+  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+}
+
+int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,
+                         const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, void* stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  if ((rc = check_heap(heap))) return rc;
+  if (variant < TCCL_S0_BULK || variant > TCCL_S2_TILEGROUP) return fail(TCCL_ERR_INVALID, "unknown variant %d", variant);
+  if ((rc = check_sync(sync, variant))) return rc;
+  const int esize = (int)dtype_size(d->out_dtype);
+  if ((rc = check_scatter(sc, d->M, d->N, esize, d->ldc, d->C))) return rc;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  build_gemm_args(d, dev, &g);
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, esize, heap, sync, tr);
+  c.op = tccl::kOpAllScatter;
+  c.directions = TCCL_DIR_PUSH;
+  c.src_col_off = sc->src_col_offset;
+  c.cols = sc->cols;
+  c.dst_ld = sc->dst_ld;
+  c.dst_col_off = sc->dst_col_offset;
+  if ((rc = set_task_units(&c, tr, false))) return rc;
+  return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+}
+
+int tccl_gemm_allgather(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap,
+                        const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, void* stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  if ((rc = check_heap(heap))) return rc;
+  if (variant < TCCL_S0_BULK || variant > TCCL_S2_TILEGROUP) return fail(TCCL_ERR_INVALID, "unknown variant %d", variant);
+  if ((rc = check_sync(sync, variant))) return rc;
+  if (!out) return fail(TCCL_ERR_INVALID, "allgather: out is NULL");
+  const int esize = (int)dtype_size(d->out_dtype);
+  if (ld_out != d->ldc) return fail(TCCL_ERR_INVALID, "allgather: ld_out must equal the GEMM's ldc");
+  const char* want = (const char*)out + (int64_t)heap->rank * d->M * ld_out * esize;
+  if ((const char*)d->C != want) return fail(TCCL_ERR_INVALID, "allgather: gemm C must point at row rank*M of out");
+  if ((d->N * esize) % 16 || (ld_out * esize) % 16) return fail(TCCL_ERR_UNSUPPORTED, "allgather: rows must be multiples of 16 bytes");
+  if (tr && !(tr->directions & (TCCL_DIR_PUSH | TCCL_DIR_PULL))) return fail(TCCL_ERR_INVALID, "allgather: no transfer direction selected");
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  build_gemm_args(d, dev, &g);
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, esize, heap, sync, tr);
+  c.op = tccl::kOpAllGather;
+  c.out = (char*)out;
+  c.ld_out_bytes = ld_out * esize;
+  if ((rc = set_task_units(&c, tr, false))) return rc;
+  return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+}
+
+int tccl_gemm_reducescatter(const tccl_gemm_desc* d, void* out, int32_t out_dtype, int64_t ld_out,
+                            const tccl_heap_view* heap, const tccl_sync_desc* sync, const tccl_transport_desc* tr,
+                            int32_t emulate_peer, int32_t variant, void* stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  if ((rc = check_heap(heap))) return rc;
+  if (variant < TCCL_S0_BULK || variant > TCCL_S2_TILEGROUP) return fail(TCCL_ERR_INVALID, "unknown variant %d", variant);
+  if ((rc = check_sync(sync, variant))) return rc;
+  if (!out || ld_out < d->N) return fail(TCCL_ERR_INVALID, "reducescatter: bad output");
+  const int esize = (int)dtype_size(d->out_dtype);
+  const int shard = d->M / heap->world_size;
+  if (d->M % heap->world_size || shard % d->block_m)
+    return fail(TCCL_ERR_INVALID, "reducescatter: M=%d must split into world_size=%d shards of whole %d-row plan tiles", d->M, heap->world_size, d->block_m);
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  build_gemm_args(d, dev, &g);
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, esize, heap, sync, tr);
+  if ((rc = fill_reduce(&c, d->C, d->out_dtype, out, out_dtype, ld_out, d->M, d->N, heap->world_size, emulate_peer))) return rc;
+  if ((rc = set_task_units(&c, tr, true))) return rc;
+  return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,431 @@
+// Communication role: the workgroups that move (or reduce) finished output while the
+// MFMA workgroups keep producing.
+//
+// Everything that is moved lives in the symmetric heap, so a location is a pair
+// (rank, byte offset inside that rank's slice); its address is heap_bases[rank] + offset
+// (reference translate_ptr: tileccl/memory/translation.py:39-99).  A transfer is a
+// rectangle of rows, cut into 16-byte units (copy) or 8-element units (reduce), and a
+// task is a contiguous range of units of one rectangle.  Each lane moves 16 bytes per
+// access (global_load_dwordx4 / global_store_dwordx4), a wavefront covers 1 KiB of a row
+// per instruction, and every thread keeps several loads in flight before its stores.
+//
+// Three operations share the machinery (reference call sites in brackets):
+//   all-scatter     column block of C -> every peer's C   [patterns/_helpers.py:86-199]
+//   all-gather      row block of `out` <-> peers' `out`   [primitives/collectives.py:613-663]
+//   reduce-scatter  out = cast(sum over ranks of partial) [primitives/collectives.py:730-783]
+// and three granularities: bulk (no waiting; the second kernel of S0), per plan tile
+// (S1: tile_wait on locks[tile]) and per TileGroup (S2: tile_wait_ge on counter[group]).
+#pragma once
+
+#include "tccl_device.h"
+
+namespace tccl {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8v __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3 };
+enum Granularity { kBulk = 0, kPerTile = 1, kPerGroup = 2 };
+enum { kDirPush = 1, kDirPull = 2 };
+enum { kF16 = 0, kBF16 = 1, kF32 = 2 };
+
+struct CommArgs {
+  int op, granularity, directions;
+  const int64_t* heap_bases;
+  int rank, world;
+  // GEMM output (C) of this rank: base, pitch, shape, element size, plan-tile geometry.
+  char* C;
+  int64_t ldc_bytes;
+  int M, N, esize;
+  int block_m, block_n, group_m, tile_rows, tile_cols, xcds, span;
+  // all-scatter placement (elements)
+  int src_col_off, cols, dst_ld, dst_col_off;
+  // all-gather: gathered output of this rank; rank r's block starts at row r*M
+  char* out;
+  int64_t ld_out_bytes;
+  // reduce-scatter: C is the partial; rs_out the owner's shard
+  char* rs_out;
+  int64_t ld_rs_out_bytes;
+  int partial_dtype, out_dtype, emulate_peer;
+  // synchronisation words and TileGroups
+  int32_t* locks;
+  int32_t* counter;
+  int32_t* barrier;
+  const int32_t* row_starts;
+  const int32_t* row_ends;
+  const int32_t* tile_counts;
+  int n_groups, epoch;
+  int32_t* trace_comm_counter;
+  int64_t* trace_ready_clock;
+  int64_t* trace_done_clock;
+  int64_t* fault;
+  int64_t spin_ticks;
+  int copy_units, reduce_units;  // units per task
+};
+
+// A rectangle to move.  Offsets are relative to a slice base.
+struct Xfer {
+  int reduce;          // 0: copy 16-byte units; 1: reduce 8-element units
+  uint32_t src_ranks;  // bit mask of slices read (copy: exactly one)
+  uint32_t dst_ranks;  // bit mask of slices written
+  int first_rank;      // reduce: the addend taken first (the owner)
+  int64_t src_off, dst_off;
+  int64_t src_pitch, dst_pitch;
+  int rows, upr;  // units per row
+};
+
+TCCL_D u32x4 ld16(const char* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+TCCL_D void st16(char* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
+
+constexpr int kThreadsComm = 256;  // threads of a communication workgroup
+constexpr int kCommUnroll = 8;     // 16-byte accesses a thread keeps in flight
+
+// ---- copy: units [u_lo, u_hi) of the rectangle, one source slice, any number of targets ----
+TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  const int tid = threadIdx.x;
+  const int src_rank = __builtin_ctz(x.src_ranks);
+  const char* src = (const char*)(uintptr_t)(a.heap_bases[src_rank] + x.src_off);
+  const bool flat = (x.src_pitch == (int64_t)x.upr * 16) && (x.dst_pitch == x.src_pitch);
+  for (int u0 = u_lo; u0 < u_hi; u0 += kThreadsComm * kCommUnroll) {
+    u32x4 v[kCommUnroll];
+    int64_t doff[kCommUnroll];
+#pragma unroll
+    for (int k = 0; k < kCommUnroll; ++k) {
+      const int u = u0 + tid + k * kThreadsComm;
+      if (u < u_hi) {
+        int64_t soff;
+        if (flat) {
+          soff = (int64_t)u * 16;
+          doff[k] = soff;
+        } else {
+          const int r = u / x.upr, c = u - r * x.upr;
+          soff = r * x.src_pitch + (int64_t)c * 16;
+          doff[k] = r * x.dst_pitch + (int64_t)c * 16;
+        }
+        v[k] = ld16(src + soff);
+      }
+    }
+    for (int q = 0; q < a.world; ++q) {
+      if (!((x.dst_ranks >> q) & 1u)) continue;
+      char* dst = (char*)(uintptr_t)(a.heap_bases[q] + x.dst_off);
+#pragma unroll
+      for (int k = 0; k < kCommUnroll; ++k) {
+        const int u = u0 + tid + k * kThreadsComm;
+        if (u < u_hi) st16(dst + doff[k], v[k]);
+      }
+    }
+  }
+}
+
+// ---- reduce: 8 elements per unit, fp32 accumulation, one rounding to the output type --------
+template <typename PT>
+TCCL_D void load8(const char* p, float (&f)[8]);
+template <>
+TCCL_D void load8<float>(const char* p, float (&f)[8]) {
+  const u32x4 a = ld16(p), b = ld16(p + 16);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    f[e] = __builtin_bit_cast(float, a[e]);
+    f[4 + e] = __builtin_bit_cast(float, b[e]);
+  }
+}
+template <>
+TCCL_D void load8<_Float16>(const char* p, float (&f)[8]) {
+  const f16x8v h = __builtin_bit_cast(f16x8v, ld16(p));
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
+}
+template <>
+TCCL_D void load8<__bf16>(const char* p, float (&f)[8]) {
+  const bf16x8v h = __builtin_bit_cast(bf16x8v, ld16(p));
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
+}
+
+template <typename OT>
+TCCL_D u32x4 pack8(const float (&f)[8]);
+template <>
+TCCL_D u32x4 pack8<_Float16>(const float (&f)[8]) {
+  f16x8v h;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = (_Float16)f[e];
+  return __builtin_bit_cast(u32x4, h);
+}
+template <>
+TCCL_D u32x4 pack8<__bf16>(const float (&f)[8]) {
+  bf16x8v h;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = (__bf16)f[e];
+  return __builtin_bit_cast(u32x4, h);
+}
+
+// Sum order: the owner's addend first, then the other ranks in ascending order
+// (tile_reduce_scatter: local chunk, then peers ascending; collectives.py:766-781).
+template <typename PT, typename OT>
+TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  constexpr int kSrcUnit = 8 * sizeof(PT);
+  const int tid = threadIdx.x;
+  const int dst_rank = __builtin_ctz(x.dst_ranks);
+  char* dst = (char*)(uintptr_t)(a.heap_bases[dst_rank] + x.dst_off);
+  const char* first = (const char*)(uintptr_t)(a.heap_bases[x.first_rank] + x.src_off);
+  for (int u = u_lo + tid; u < u_hi; u += kThreadsComm) {
+    const int r = u / x.upr, c = u - r * x.upr;
+    const int64_t soff = r * x.src_pitch + (int64_t)c * kSrcUnit;
+    float acc[8];
+    load8<PT>(first + soff, acc);
+    for (int p = 0; p < a.world; ++p) {
+      if (p == x.first_rank || !((x.src_ranks >> p) & 1u)) continue;
+      float in[8];
+      load8<PT>((const char*)(uintptr_t)(a.heap_bases[p] + x.src_off) + soff, in);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += in[e];
+    }
+    st16(dst + r * x.dst_pitch + (int64_t)c * 16, pack8<OT>(acc));
+  }
+}
+
+TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  const int key = a.partial_dtype * 4 + a.out_dtype;
+  switch (key) {
+    case kF32 * 4 + kF16: run_reduce_t<float, _Float16>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kBF16: run_reduce_t<float, __bf16>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kF16: run_reduce_t<_Float16, _Float16>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16>(a, x, u_lo, u_hi); break;
+    default: break;
+  }
+}
+
+TCCL_D void run_xfer(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  if (x.reduce)
+    run_reduce(a, x, u_lo, u_hi);
+  else
+    run_copy(a, x, u_lo, u_hi);
+}
+
+// ---- rectangles of the three operations ----------------------------------------------------------
+// `peer` is the other party of a pull (the slice read); pushes fan out to all peers.
+// Rows [r0, r1) and columns [c0, c1) are relative to this rank's GEMM output C.
+TCCL_D uint32_t all_ranks(int world) { return world >= 32 ? 0xffffffffu : ((1u << world) - 1u); }
+
+TCCL_D int64_t slice_offset(const CommArgs& a, const char* p) { return (int64_t)(uintptr_t)p - a.heap_bases[a.rank]; }
+
+// Returns false when the rectangle is empty.
+TCCL_D bool make_xfer(const CommArgs& a, bool pull, int peer, int r0, int r1, int c0, int c1, Xfer& x) {
+  if (r1 > a.M) r1 = a.M;
+  if (c1 > a.N) c1 = a.N;
+  x.reduce = 0;
+  x.first_rank = a.rank;
+  if (a.op == kOpAllScatter) {
+    // Only columns inside [src_col_off, src_col_off + cols) travel (_helpers.py:148-151).
+    const int lo = c0 > a.src_col_off ? c0 : a.src_col_off;
+    const int hi = c1 < a.src_col_off + a.cols ? c1 : a.src_col_off + a.cols;
+    if (lo >= hi || r0 >= r1) return false;
+    const int64_t c_off = slice_offset(a, a.C);
+    x.src_ranks = 1u << a.rank;
+    x.dst_ranks = all_ranks(a.world) & ~(1u << a.rank);
+    x.src_pitch = a.ldc_bytes;
+    x.dst_pitch = (int64_t)a.dst_ld * a.esize;
+    x.src_off = c_off + r0 * x.src_pitch + (int64_t)lo * a.esize;
+    x.dst_off = c_off + r0 * x.dst_pitch + (int64_t)(a.dst_col_off + lo - a.src_col_off) * a.esize;
+    x.rows = r1 - r0;
+    x.upr = (hi - lo) * a.esize / 16;
+    return x.dst_ranks != 0;
+  }
+  if (r0 >= r1 || c0 >= c1) return false;
+  if (a.op == kOpAllGather) {
+    // Block of rank b sits at rows [b*M, (b+1)*M) of every rank's `out` (collectives.py:628-630).
+    const int owner = pull ? peer : a.rank;
+    const int64_t off = slice_offset(a, a.out) + ((int64_t)owner * a.M + r0) * a.ld_out_bytes + (int64_t)c0 * a.esize;
+    x.src_ranks = 1u << owner;
+    x.dst_ranks = pull ? (1u << a.rank) : (all_ranks(a.world) & ~(1u << a.rank));
+    x.src_off = x.dst_off = off;
+    x.src_pitch = x.dst_pitch = a.ld_out_bytes;
+    x.rows = r1 - r0;
+    x.upr = (c1 - c0) * a.esize / 16;
+    return x.dst_ranks != 0;
+  }
+  // Reduce-scatter: rows belong to owner = row / (M / world); the owner's shard is rs_out.
+  const int shard = a.M / a.world;
+  const int owner = r0 / shard;
+  if (owner != a.rank && !a.emulate_peer) return false;
+  const int out_esize = 2;
+  x.reduce = 1;
+  x.first_rank = owner;
+  x.src_ranks = all_ranks(a.world);
+  x.dst_ranks = 1u << owner;
+  x.src_pitch = a.ldc_bytes;
+  x.dst_pitch = a.ld_rs_out_bytes;
+  x.src_off = slice_offset(a, a.C) + r0 * x.src_pitch + (int64_t)c0 * a.esize;
+  x.dst_off = slice_offset(a, a.rs_out) + (int64_t)(r0 - owner * shard) * x.dst_pitch + (int64_t)c0 * out_esize;
+  x.rows = r1 - r0;
+  x.upr = (c1 - c0) / 8;
+  return true;
+}
+
+// ---- waiting -------------------------------------------------------------------------------------
+// One lane spins; the verdict is shared through one LDS word.  Returns false on timeout,
+// after raising *fault, so that every workgroup still runs to its end.
+struct Waiter {
+  const CommArgs& a;
+  volatile int* verdict;
+  int64_t deadline;
+
+  TCCL_D bool finish(bool ok) const {
+    if (threadIdx.x == 0) {
+      if (!ok && a.fault) *a.fault = 1;
+      *verdict = ok ? 1 : 0;
+    }
+    __syncthreads();
+    const bool all_ok = *verdict != 0;
+    __syncthreads();
+    observe_fence();
+    return all_ok;
+  }
+
+  // S1: locks[tile] of `rank`'s slice.  Own locks are consumed (tile_wait); a peer's are
+  // only observed (tile_poll), since the peer's own workgroups consume them.
+  TCCL_D bool tile(int tile_id, int rank) const {
+    bool ok = true;
+    if (threadIdx.x == 0) {
+      int32_t* w = translate_ptr(a.locks, a.rank, rank, a.heap_bases);
+      ok = tile_wait(w, tile_id, /*consume=*/rank == a.rank, deadline);
+    }
+    return finish(ok);
+  }
+
+  // S2: counter[g] of every slice in `ranks` has reached epoch * tile_counts[g].
+  TCCL_D bool group(int g, uint32_t ranks) const {
+    bool ok = true;
+    if (threadIdx.x == 0) {
+      const int32_t need = a.epoch * a.tile_counts[g];
+      for (int r = 0; r < a.world && ok; ++r)
+        if ((ranks >> r) & 1u) ok = tile_wait_ge(translate_ptr(a.counter, a.rank, r, a.heap_bases), g, need, deadline);
+      if (ok && a.trace_ready_clock) {
+        unsigned long long* slot = (unsigned long long*)&a.trace_ready_clock[g];
+        atomicCAS(slot, 0ull, (unsigned long long)now_ticks());
+      }
+    }
+    return finish(ok);
+  }
+};
+
+// A finished task of group g: count it; the task that completes the group stamps the clock.
+TCCL_D void task_done(const CommArgs& a, int g, int tasks_of_group) {
+  publish_fence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (a.trace_comm_counter) atomicAdd(&a.trace_comm_counter[g], 1);
+    if (a.barrier) {
+      const int32_t prev = tile_signal_add(a.barrier, g, 1);
+      if (prev + 1 == a.epoch * tasks_of_group && a.trace_done_clock) a.trace_done_clock[g] = now_ticks();
+    }
+  }
+}
+
+TCCL_D int cdiv(int x, int y) { return (x + y - 1) / y; }
+
+// Without a plan (row_starts == nullptr) the whole output is one group; for a
+// reduce-scatter it is one group per owner shard, so no task straddles two owners.
+TCCL_D int group_lo(const CommArgs& a, int g) {
+  if (a.row_starts) return a.row_starts[g];
+  return a.op == kOpReduceScatter ? g * (a.M / a.world) : 0;
+}
+TCCL_D int group_hi(const CommArgs& a, int g) {
+  if (a.row_ends) return a.row_ends[g];
+  return a.op == kOpReduceScatter ? (g + 1) * (a.M / a.world) : a.M;
+}
+// Reduce-scatter rows this rank neither owns nor reduces on the owner's behalf.
+TCCL_D bool rs_not_mine(const CommArgs& a, int row) {
+  return a.op == kOpReduceScatter && !a.emulate_peer && row / (a.M / a.world) != a.rank;
+}
+
+// ---- the role ---------------------------------------------------------------------------------------
+// Tasks are numbered so that whatever can start earliest comes first: pulls (their
+// sources are ready or soon will be, independent of this rank's GEMM), then pushes /
+// reductions in production order.  Workgroup w takes tasks w, w + n, w + 2n, ...; no
+// GEMM workgroup ever waits on a communication workgroup, so the order is deadlock-free.
+TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
+  if (a.op == kOpNone || num_wgs <= 0) return;
+  Waiter wait{a, lds_word, now_ticks() + a.spin_ticks};
+  const int peers = a.world - 1;
+  const bool is_rs = a.op == kOpReduceScatter;
+  const bool do_pull = !is_rs && a.op == kOpAllGather && (a.directions & kDirPull) && peers > 0;
+  const bool do_push = is_rs || (a.directions & kDirPush);
+  const int unit_elems = is_rs ? 8 : 16 / a.esize;
+  const int units_per_task = is_rs ? a.reduce_units : a.copy_units;
+
+  if (a.granularity == kPerTile) {
+    const int total = a.tile_rows * a.tile_cols;
+    const int n_pull = do_pull ? peers * total : 0;
+    const int n_all = n_pull + (do_push ? total : 0);
+    for (int t = wg; t < n_all; t += num_wgs) {
+      const bool pull = t < n_pull;
+      const int local = pull ? t % total : t - n_pull;
+      int peer = a.rank;
+      if (pull) {
+        peer = t / total;
+        if (peer >= a.rank) ++peer;
+      }
+      const int tile_id = tile_for_slot(local, total, a.xcds, a.span);
+      const TileCoord tc = tile_coords(tile_id, a.tile_rows, a.tile_cols, a.group_m);
+      bool ok;
+      if (pull) {
+        ok = wait.tile(tile_id, peer);
+      } else {
+        ok = wait.tile(tile_id, a.rank);
+        if (is_rs)  // the peers' partial tiles must be there as well
+          for (int p = 0; p < a.world && ok; ++p)
+            if (p != a.rank) ok = wait.tile(tile_id, p);
+      }
+      Xfer x;
+      const int r0 = tc.m * a.block_m, c0 = tc.n * a.block_n;
+      if (ok && make_xfer(a, pull, peer, r0, r0 + a.block_m, c0, c0 + a.block_n, x)) run_xfer(a, x, 0, x.rows * x.upr);
+    }
+    return;
+  }
+
+  // Bulk and per-group: tasks are ranges of units_per_task units of a group's rectangle
+  // (bulk treats the plan's groups as plain work partitions and never waits).
+  const int row_units = is_rs ? a.N / 8 : (a.op == kOpAllScatter ? a.cols : a.N) / unit_elems;
+  int total = 0;
+  for (int g = 0; g < a.n_groups; ++g) total += cdiv((group_hi(a, g) - group_lo(a, g)) * row_units, units_per_task);
+  const int n_pull = do_pull ? peers * total : 0;
+  const int n_all = n_pull + (do_push ? total : 0);
+  const int tasks_factor = (do_pull ? peers : 0) + (do_push ? 1 : 0);
+  for (int t = wg; t < n_all; t += num_wgs) {
+    const bool pull = t < n_pull;
+    int local = pull ? t % total : t - n_pull;
+    int peer = a.rank;
+    if (pull) {
+      peer = t / total;
+      if (peer >= a.rank) ++peer;
+    }
+    int g = 0, tasks_g = 0;
+    for (; g < a.n_groups; ++g) {
+      tasks_g = cdiv((group_hi(a, g) - group_lo(a, g)) * row_units, units_per_task);
+      if (local < tasks_g) break;
+      local -= tasks_g;
+    }
+    if (g >= a.n_groups) break;
+    if (rs_not_mine(a, group_lo(a, g))) continue;
+    bool ok = true;
+    if (a.granularity == kPerGroup) {
+      uint32_t ranks = pull ? (1u << peer) : (is_rs ? all_ranks(a.world) : (1u << a.rank));
+      ok = wait.group(g, ranks);
+    }
+    Xfer x;
+    if (ok && make_xfer(a, pull, peer, group_lo(a, g), group_hi(a, g), 0, a.N, x)) {
+      const int units = x.rows * x.upr;
+      const int lo = local * units_per_task;
+      const int hi = lo + units_per_task < units ? lo + units_per_task : units;
+      if (lo < hi) run_xfer(a, x, lo, hi);
+    }
+    if (a.granularity == kPerGroup) task_done(a, g, tasks_g * tasks_factor);
+  }
+}
+
+}  // namespace tccl

@@ -1,0 +1,135 @@
+// Device-side primitives shared by every kernel of libtileccl_hip: index math of the
+// persistent GEMM's tile order, symmetric-heap pointer translation, and the
+// signal / wait words.  Index helpers are __host__ __device__ so CPU tests can call the
+// very code the kernels run.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define TCCL_HD __host__ __device__ __forceinline__
+#define TCCL_D __device__ __forceinline__
+
+namespace tccl {
+
+// ---------------------------------------------------------------------------------------
+// Tile order.  Swizzled tile id -> (tile_m, tile_n): inside a band of group_m tile rows
+// (fewer in the last band) ids walk down the rows first, then across the columns.
+// Reference: tileccl/kernels/gemm.py:118-123, tileccl_v2/tile_group.py:229-234.
+// ---------------------------------------------------------------------------------------
+struct TileCoord {
+  int m, n;
+};
+
+TCCL_HD TileCoord tile_coords(int tile_id, int tile_rows, int tile_cols, int group_m) {
+  const int per_band = group_m * tile_cols;
+  const int band = tile_id / per_band;
+  const int first_m = band * group_m;
+  const int height = (tile_rows - first_m) < group_m ? (tile_rows - first_m) : group_m;
+  const int within = tile_id - band * per_band;
+  TileCoord c;
+  c.m = first_m + within % height;
+  c.n = within / height;
+  return c;
+}
+
+// Inverse of tile_coords.
+TCCL_HD int tile_id_of(int tile_m, int tile_n, int tile_rows, int tile_cols, int group_m) {
+  const int band = tile_m / group_m;
+  const int first_m = band * group_m;
+  const int height = (tile_rows - first_m) < group_m ? (tile_rows - first_m) : group_m;
+  return band * group_m * tile_cols + tile_n * height + (tile_m - first_m);
+}
+
+// Launch slot -> tile id.  Workgroups are handed to the XCDs round-robin (slot % xcds),
+// and each XCD has a private L2.  Inside every full block of xcds*span consecutive tile
+// ids, XCD x takes the ids [x*span, (x+1)*span): with the row-fastest swizzle that is a
+// compact patch of the output (span/group_m tile columns of one band), so the A rows and
+// B columns it touches stay in that XCD's L2.  A trailing partial block keeps the
+// identity order.  The map is a bijection on [0, total_tiles).
+TCCL_HD int tile_for_slot(int slot, int total_tiles, int xcds, int span) {
+  const int block = xcds * span;
+  const int base = (slot / block) * block;
+  if (xcds <= 1 || base + block > total_tiles) return slot;
+  const int r = slot - base;
+  return base + (r % xcds) * span + r / xcds;
+}
+
+#ifdef __HIPCC__
+// ---------------------------------------------------------------------------------------
+// Symmetric heap.  translate(ptr, from, to) = bases[to] + (ptr - bases[from]).
+// Reference: tileccl/memory/translation.py:39-99, tileccl_v2/ipc.py:24-63.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+TCCL_D T* translate_ptr(T* ptr, int from_rank, int to_rank, const int64_t* heap_bases) {
+  const int64_t off = (int64_t)(uintptr_t)ptr - heap_bases[from_rank];
+  return (T*)(uintptr_t)(heap_bases[to_rank] + off);
+}
+
+// 100 MHz constant clock; one tick = 10 ns.
+TCCL_D int64_t now_ticks() { return (int64_t)wall_clock64(); }
+
+// ---------------------------------------------------------------------------------------
+// Signal words (int32, in the heap).  One GPU: agent scope is enough for every
+// workgroup on every XCD to observe a release; real peers would need system scope
+// (the reference's v1 default is "gpu", v2 "sys": sync/primitives.py:357, ipc.py:137).
+// ---------------------------------------------------------------------------------------
+
+// tile_signal: locks[i] = 1, release.  (sync/primitives.py:357-387)
+TCCL_D void tile_signal(int32_t* locks, int i) {
+  __hip_atomic_exchange(&locks[i], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One CAS probe: consuming (1 -> 0, tile_wait / tile_try_wait) or non-consuming
+// (1 -> 1, tile_poll / tile_try_poll).  (sync/primitives.py:390-439, ipc.py:193-228)
+TCCL_D bool tile_probe(int32_t* locks, int i, bool consume) {
+  int32_t expected = 1;
+  return __hip_atomic_compare_exchange_strong(&locks[i], &expected, consume ? 0 : 1, __ATOMIC_ACQUIRE,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// tile_try_wait / tile_try_poll: at most max_spins probes; true when the flag was seen.
+TCCL_D bool tile_try_wait(int32_t* locks, int i, int max_spins, bool consume) {
+  for (int s = 0; s < max_spins; ++s)
+    if (tile_probe(locks, i, consume)) return true;
+  return false;
+}
+
+// tile_wait / tile_poll with a deadline: the reference spins forever
+// (sync/primitives.py:390-414); here every wait gives up at `deadline` (now_ticks units)
+// and reports false so the kernel can drain and the host can raise.
+TCCL_D bool tile_wait(int32_t* locks, int i, bool consume, int64_t deadline) {
+  for (;;) {
+    if (tile_try_wait(locks, i, 64, consume)) return true;
+    if (now_ticks() > deadline) return false;
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
+// tile_signal_add: counter[i] += v, release; returns the previous value. (ipc.py:231-241)
+TCCL_D int32_t tile_signal_add(int32_t* words, int i, int32_t v) {
+  return __hip_atomic_fetch_add(&words[i], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// tile_wait_ge: spin until counter[i] >= threshold (acquire).  The reference reads the
+// word with atomic_add(0) (ipc.py:244-254); an acquire load observes the same value
+// without taking the line exclusive.  Bounded like tile_wait.
+TCCL_D bool tile_wait_ge(const int32_t* words, int i, int32_t threshold, int64_t deadline) {
+  for (;;) {
+    for (int s = 0; s < 32; ++s) {
+      if (__hip_atomic_load(&words[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) >= threshold) return true;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (now_ticks() > deadline) return false;
+  }
+}
+
+// Every thread of the workgroup has finished its global stores -> make them visible at
+// agent scope before one thread publishes the signal.
+TCCL_D void publish_fence() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
+// After one thread's acquire-wait and a workgroup barrier, every other thread drops
+// stale cache lines before reading the signalled data.
+TCCL_D void observe_fence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+#endif  // __HIPCC__
+
+}  // namespace tccl
