@@ -1,0 +1,109 @@
+"""CPU restatement of the fused GEMM + collective semantics (test infrastructure only).
+
+All arithmetic is torch on the CPU.  Follows
+    GEMM: fp32 accumulate, one cast to the output type
+        /root/reference/tileccl/kernels/gemm.py:139-167, patterns/bulk_sync.py:213-238
+    scatter placement of a tile into a peer's C
+        /root/reference/tileccl/patterns/_helpers.py:145-157
+    fan-out to every peer but self
+        /root/reference/tileccl/patterns/_helpers.py:161-199
+    all-gather layout [block_rank0 | block_rank1 | ...]
+        /root/reference/tileccl/primitives/collectives.py:628-663
+    reduce-scatter: owner's chunk first, then peers ascending
+        /root/reference/tileccl/primitives/collectives.py:766-783
+    (this build accumulates the reduction in fp32 and rounds once, as its north star asks;
+     the reference accumulates in the tensor dtype)
+"""
+
+from __future__ import annotations
+
+import torch
+
+
+def gemm(A: torch.Tensor, B: torch.Tensor, out_dtype: torch.dtype, alpha: float = 1.0) -> torch.Tensor:
+    """``cast(alpha * (A.float() @ B.float()))``; fp8 inputs are dequantised exactly by ``.float()``."""
+    acc = A.float() @ B.float()
+    if alpha != 1.0:
+        acc = acc * alpha
+    return acc.to(out_dtype)
+
+
+def scatter_into_peer(peer_C: torch.Tensor, local_C: torch.Tensor, src_col_offset: int, cols: int,
+                      dst_ld: int, dst_col_offset: int) -> None:
+    """Vectorised placement: peer_flat[r*dst_ld + dst_col_offset + j] = local_C[r, src_col_offset + j]."""
+    M = local_C.shape[0]
+    flat = peer_C.reshape(-1)
+    rows = torch.arange(M).unsqueeze(1) * dst_ld
+    js = torch.arange(cols).unsqueeze(0)
+    flat[(rows + dst_col_offset + js).reshape(-1)] = local_C[:, src_col_offset:src_col_offset + cols].reshape(-1)
+
+
+def scatter_into_peer_by_tiles(peer_C, local_C, src_col_offset, cols, dst_ld, dst_col_offset,
+                               block_m=128, block_n=128) -> None:
+    """Element loop over tiles with the reference's mask, for small cases (_helpers.py:148-157)."""
+    M, N = local_C.shape
+    flat = peer_C.reshape(-1)
+    for tm in range(-(-M // block_m)):
+        for tn in range(-(-N // block_n)):
+            for r in range(tm * block_m, min((tm + 1) * block_m, M)):
+                for c in range(tn * block_n, min((tn + 1) * block_n, N)):
+                    if src_col_offset <= c < src_col_offset + cols:
+                        flat[r * dst_ld + dst_col_offset + (c - src_col_offset)] = local_C[r, c]
+
+
+def gemm_allscatter(As, Bs, Cs, specs) -> None:
+    """All ranks of one process: every rank computes its C, then scatters to every peer.
+
+    ``specs[r]`` carries the four placement integers of rank ``r``; ranks run in rank order,
+    like sequential single-process launches do.
+    """
+    world = len(As)
+    for r in range(world):
+        Cs[r].copy_(gemm(As[r], Bs[r], Cs[r].dtype))
+        s = specs[r]
+        for p in range(world):
+            if p != r:
+                scatter_into_peer(Cs[p], Cs[r], s["src_col_offset"], s["cols"], s["dst_ld"], s["dst_col_offset"])
+
+
+def allgather_exchange(outs, rank: int, M: int, push: bool = True, pull: bool = True) -> None:
+    """Rank's own block goes to every peer (push); every peer's block comes in (pull)."""
+    world = len(outs)
+    for p in range(world):
+        if p == rank:
+            continue
+        if push:
+            outs[p][rank * M:(rank + 1) * M] = outs[rank][rank * M:(rank + 1) * M]
+        if pull:
+            outs[rank][p * M:(p + 1) * M] = outs[p][p * M:(p + 1) * M]
+
+
+def gemm_allgather(A, B, outs, rank: int, push: bool = True, pull: bool = True, alpha: float = 1.0) -> None:
+    M = A.shape[0]
+    outs[rank][rank * M:(rank + 1) * M] = gemm(A, B, outs[rank].dtype, alpha)
+    allgather_exchange(outs, rank, M, push, pull)
+
+
+def reduce_rows(partials, owner: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """Owner's shard: fp32 sum, owner first then the other ranks ascending, one rounding."""
+    world = len(partials)
+    shard = partials[0].shape[0] // world
+    lo, hi = owner * shard, (owner + 1) * shard
+    acc = partials[owner][lo:hi].float().clone()
+    for p in range(world):
+        if p != owner:
+            acc += partials[p][lo:hi].float()
+    return acc.to(out_dtype)
+
+
+def gemm_reducescatter(A, B, partials, outs, rank: int, emulate_peer: bool = True, alpha: float = 1.0) -> None:
+    """partials[rank] = A@B (partial dtype); outs[o] = reduce(owner o) for the owners handled."""
+    partials[rank].copy_(gemm(A, B, partials[rank].dtype, alpha))
+    for owner in range(len(partials)):
+        if owner == rank or emulate_peer:
+            outs[owner].copy_(reduce_rows(partials, owner, outs[owner].dtype))
+
+
+def expected_counters(tile_counts, epoch: int = 1):
+    """counter[g] after ``epoch`` launches without reset: every tile of the group signalled once each."""
+    return [epoch * t for t in tile_counts]

@@ -1,0 +1,152 @@
+"""PatternExecutionSpec placement and the public gemm_allscatter contract: closed forms and
+error messages (reference tileccl/patterns/contracts.py, tileccl/ops.py:1306-1404)."""
+
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from tileccl_amd.patterns.contracts import resolve_pattern_execution
+from tileccl_amd.patterns.runtime import resolve_dual_role_scheduler
+
+
+def T(rows, cols):
+    return torch.empty(rows, cols, dtype=torch.float16)
+
+
+def test_full_full_two_ranks_is_baseline_config_0():
+    for rank in (0, 1):
+        s = resolve_pattern_execution(T(512, 256), T(256, 512), T(512, 512), rank=rank, world_size=2,
+                                      b_layout="full", c_layout="full")
+        assert (s.M, s.K, s.full_N, s.local_N) == (512, 256, 512, 512)
+        assert s.scatter_cols == 256
+        assert s.scatter_src_col_offset == s.scatter_dst_col_offset == rank * 256
+        assert s.scatter_dst_leading_dim == 512
+        assert s.rhs_layout == s.output_layout == "full"
+        assert s.rhs.full_shape == (256, 512) and s.output.local_shape == (512, 512)
+        d = s.to_dict()
+        assert d["scatter"] == {"src_col_offset": rank * 256, "cols": 256, "dst_leading_dim": 512, "dst_col_offset": rank * 256}
+        assert d["rhs"]["layout_kind"] == "full" and d["output"]["full_shape"] == [512, 512]
+
+
+def test_single_rank_scatters_everything_nowhere():
+    s = resolve_pattern_execution(T(128, 64), T(64, 128), T(128, 128), rank=0, world_size=1)
+    assert (s.scatter_cols, s.scatter_src_col_offset, s.scatter_dst_col_offset, s.scatter_dst_leading_dim) == (128, 0, 0, 128)
+    assert s.output_layout == "full"
+
+
+def test_shard_shard():
+    s = resolve_pattern_execution(T(64, 32), T(32, 100), T(64, 100), rank=3, world_size=4, full_N=400,
+                                  b_layout="shard", c_layout="shard")
+    assert (s.full_N, s.local_N, s.scatter_cols, s.scatter_src_col_offset, s.scatter_dst_col_offset,
+            s.scatter_dst_leading_dim) == (400, 100, 100, 0, 0, 100)
+    assert s.output.cols == 100 and s.rhs.layout_kind == "shard"
+    # full_N implied by the hints
+    s2 = resolve_pattern_execution(T(64, 32), T(32, 100), T(64, 100), rank=0, world_size=4,
+                                   b_layout="shard", c_layout="shard")
+    assert s2.full_N == 400
+
+
+def test_layout_inference_without_hints():
+    # mixed widths (hi == lo*world) pin full_N, but mixed layouts are then rejected
+    with pytest.raises(ValueError, match="Mixed multi-rank layouts are not implemented yet"):
+        resolve_pattern_execution(T(8, 8), T(8, 64), T(8, 32), rank=0, world_size=2)
+    with pytest.raises(ValueError, match="Ambiguous multi-rank pattern contract"):
+        resolve_pattern_execution(T(8, 8), T(8, 64), T(8, 64), rank=0, world_size=2)
+    s = resolve_pattern_execution(T(8, 8), T(8, 64), T(8, 64), rank=1, world_size=2, full_N=64)
+    assert s.output_layout == "full" and s.scatter_src_col_offset == 32
+    s = resolve_pattern_execution(T(8, 8), T(8, 64), T(8, 64), rank=1, world_size=2, full_N=128)
+    assert s.output_layout == "shard"
+
+
+@pytest.mark.parametrize(
+    "args,kw,msg",
+    [
+        ((torch.empty(2, 2, 2), T(2, 2), T(2, 2)), dict(rank=0, world_size=1), "Pattern tensors must all be 2-D: got A.ndim=3"),
+        ((T(2, 2), T(2, 2), T(2, 2)), dict(rank=0, world_size=0), "world_size must be >= 1, got 0"),
+        ((T(2, 2), T(2, 2), T(2, 2)), dict(rank=2, world_size=2), "rank=2 out of range for world_size=2"),
+        ((T(2, 3), T(2, 2), T(2, 2)), dict(rank=0, world_size=1), r"B.shape\[0\] must equal A.shape\[1\]: got 2 vs 3"),
+        ((T(2, 2), T(2, 2), T(3, 2)), dict(rank=0, world_size=1), r"C.shape\[0\] must equal A.shape\[0\]: got 3 vs 2"),
+        ((T(2, 2), T(2, 2), T(2, 2)), dict(rank=0, world_size=1, b_layout="diag"), r"b_layout must be one of \['full', 'shard'\], got 'diag'"),
+        ((T(2, 2), T(2, 8), T(2, 8)), dict(rank=0, world_size=2, full_N=9, b_layout="full", c_layout="full"),
+         r"full_N must be divisible by world_size: 9 % 2 != 0"),
+        ((T(2, 2), T(2, 8), T(2, 8)), dict(rank=0, world_size=2, full_N=0), "full_N must be positive, got 0"),
+        ((T(2, 2), T(2, 8), T(2, 4)), dict(rank=0, world_size=2, b_layout="full", c_layout="full"),
+         r"Provided layout hints disagree on full_N: resolved candidates=\[4, 8\]"),
+        ((T(2, 2), T(2, 6), T(2, 6)), dict(rank=0, world_size=2, full_N=8, b_layout="full", c_layout="full"),
+         "B layout='full' expects 8 columns, got 6"),
+        ((T(2, 2), T(2, 6), T(2, 6)), dict(rank=0, world_size=2, full_N=8), "Cannot infer B layout from cols=6, full_N=8, shard_N=4"),
+        ((T(2, 2), T(2, 6), T(2, 6)), dict(rank=0, world_size=1, full_N=8), "B expects 8 columns, got 6"),
+    ],
+)
+def test_contract_errors(args, kw, msg):
+    with pytest.raises(ValueError, match=msg):
+        resolve_pattern_execution(*args, **kw)
+
+
+def test_dual_role_scheduler():
+    s = resolve_dual_role_scheduler(256)
+    assert (s.compute_sms, s.comm_sms, s.policy) == (205, 51, "fractional_split")
+    s = resolve_dual_role_scheduler(132)
+    assert (s.compute_sms, s.comm_sms) == (106, 26)
+    s = resolve_dual_role_scheduler(2, comm_sm_fraction=0.99)
+    assert (s.compute_sms, s.comm_sms) == (1, 1)
+    s = resolve_dual_role_scheduler(256, compute_sms=200, comm_sms=40)
+    assert (s.compute_sms, s.comm_sms, s.policy) == (200, 40, "explicit")
+    with pytest.raises(ValueError, match="requires at least 2 compute units"):
+        resolve_dual_role_scheduler(1)
+    with pytest.raises(ValueError, match="requires both compute_sms and comm_sms to be > 0"):
+        resolve_dual_role_scheduler(256, compute_sms=10)
+    with pytest.raises(ValueError, match=r"cannot exceed the device SM count: 200 \+ 100 > 256"):
+        resolve_dual_role_scheduler(256, compute_sms=200, comm_sms=100)
+
+
+# ---- public op contract, exercised with a stand-in context on CPU tensors ---------------------------------
+def fake_ctx(rank=0, world_size=2):
+    return SimpleNamespace(rank=rank, world_size=world_size, device="cpu", backend_name="hip",
+                           require_heap=lambda: object())
+
+
+def test_public_layout_defaults_and_contract():
+    from tileccl_amd import ops
+
+    assert ops._resolve_public_layout_contract(b_layout=None, c_layout=None) == ("full", "full")
+    with pytest.raises(ValueError, match="b_layout and c_layout must be specified together"):
+        ops._resolve_public_layout_contract(b_layout="full", c_layout=None)
+    k = ops._resolve_gemm_allscatter_contract(T(512, 256), T(256, 512), T(512, 512), ctx=fake_ctx(1), full_N=None,
+                                              b_layout="full", c_layout="full", storage_kind="symmetric")
+    assert k.to_dict() == dict(M=512, K=256, full_N=512, rhs_cols=512, output_cols=512, rank=1, world_size=2,
+                               rhs_layout="full", output_layout="full", storage_kind="symmetric")
+    k = ops._resolve_gemm_allscatter_contract(T(8, 8), T(8, 64), T(8, 32), ctx=fake_ctx(), full_N=None,
+                                              b_layout="full", c_layout="shard", storage_kind="symmetric")
+    assert (k.full_N, k.rhs_cols, k.output_cols) == (64, 64, 32)
+    with pytest.raises(ValueError, match="gemm_allscatter tensors must all reside on the context device cuda:0"):
+        bad = fake_ctx()
+        bad.device = "cuda:0"
+        ops._resolve_gemm_allscatter_contract(T(8, 8), T(8, 8), T(8, 8), ctx=bad, full_N=None, b_layout="full",
+                                              c_layout="full", storage_kind="symmetric")
+    with pytest.raises(ValueError, match="C layout='full' expects 64 columns, got 32"):
+        ops._resolve_gemm_allscatter_contract(T(8, 8), T(8, 64), T(8, 32), ctx=fake_ctx(), full_N=64,
+                                              b_layout="full", c_layout="full", storage_kind="symmetric")
+
+
+def test_pattern_resolution_by_name_class_instance():
+    from tileccl_amd import ops
+    from tileccl_amd.patterns import BulkSyncPattern, TileGroupPattern, WGSpecializedPattern
+
+    ctx = fake_ctx()
+    spec = resolve_pattern_execution(T(8, 8), T(8, 8), T(8, 8), rank=0, world_size=2, b_layout="full", c_layout="full")
+    pick = lambda p: ops._resolve_pattern_impl(pattern=p, ctx=ctx, execution=spec, hw_info=None)  # noqa: E731
+    assert isinstance(pick("bulk_sync"), BulkSyncPattern) and isinstance(pick("wg_spec"), WGSpecializedPattern)
+    assert isinstance(pick("s2"), TileGroupPattern) and isinstance(pick("auto"), TileGroupPattern)
+    assert isinstance(pick(BulkSyncPattern), BulkSyncPattern)
+    inst = WGSpecializedPattern(ctx)
+    assert pick(inst) is inst
+    with pytest.raises(ValueError, match="Unknown pattern 'warp_drive'"):
+        pick("warp_drive")
+    with pytest.raises(TypeError, match="pattern must be a pattern name"):
+        pick(3.5)
+    with pytest.raises(ValueError, match="Pattern instance rank does not match the provided context: 1 != 0"):
+        pick(WGSpecializedPattern(fake_ctx(rank=1)))
+    with pytest.raises(ValueError, match="BLOCK_K=32"):
+        BulkSyncPattern(ctx, BLOCK_K=32)

@@ -1,0 +1,173 @@
+"""GEMM-output AllGather (Gate 1) in the S0 / S1 / S2 variants against the CPU oracle.
+
+Placement and copied bytes must be bit-exact against the GEMM output; the GEMM itself is
+held to the fp32-matmul tolerance.  Full-size BASELINE configs are covered through
+size-independent properties (both slices end identical, idempotence, counters)."""
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import assert_gemm_close, bits, into_heap, seeded
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = ["s0", "s1", "s2"]
+
+
+def make(world, M, N, dtype=torch.float16, heap_bytes=256 << 20, **kw):
+    from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(heap_bytes, world)
+    ops = [FusedGemmAllGather(h, M, N, dtype, **kw) for h in heaps]
+    return heaps, ops
+
+
+def fill_peer_blocks(ops, M, N, dtype, seed=2):
+    """Each peer's own row block is a seeded N(0,1) tensor resident in its slice."""
+    blocks = {}
+    for p, op in enumerate(ops):
+        if p == 0:
+            continue
+        blocks[p] = seeded((M, N), seed + p, dtype)
+        op.out.zero_()
+        op.out[p * M:(p + 1) * M].copy_(blocks[p])
+    return blocks
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("directions", ["both", "push", "pull"])
+def test_small_two_ranks_against_oracle(lib, variant, directions):
+    M, N, K = 512, 512, 256
+    heaps, ops = make(2, M, N, directions=directions)
+    try:
+        op = ops[0]
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        blocks = fill_peer_blocks(ops, M, N, torch.float16)
+        op.out.zero_()
+        op.mark_peers_ready()
+        op(A, B, variant)
+        op.check_faults()
+        # oracle on identical bits: slices as CPU tensors
+        outs = [torch.zeros(2 * M, N, dtype=torch.float16) for _ in range(2)]
+        outs[1][M:] = blocks[1]
+        oracle.gemm_allgather(A_cpu, B_cpu, outs, 0, push=directions != "pull", pull=directions != "push")
+        mine = op.out[:M].clone()
+        assert_gemm_close(mine, A_cpu.float() @ B_cpu.float(), tight=0.004)
+        assert (mine.cpu().float() - outs[0][:M].float()).abs().max().item() <= 0.004
+        # everything that was *moved* is bit-exact
+        if directions != "pull":
+            assert torch.equal(bits(op.peer_out(1)[:M]), bits(mine))
+        else:
+            assert torch.count_nonzero(op.peer_out(1)[:M]).item() == 0  # nothing pushed
+        if directions != "push":
+            assert torch.equal(bits(op.out[M:]).cpu(), bits(blocks[1]))
+        else:
+            assert torch.count_nonzero(op.out[M:]).item() == 0  # nothing pulled
+        assert torch.equal(bits(op.peer_out(1)[M:]).cpu(), bits(blocks[1]))  # the peer's own block is untouched
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_ragged_shape_four_ranks_many_groups(lib, variant):
+    """M not a multiple of the tile, several groups per rank, fan-out to three peers."""
+    M, N, K = 1000, 264, 72
+    heaps, ops = make(4, M, N, dtype=torch.bfloat16, tau_min_bytes=1, group_m=2,
+                      transport=__import__("tileccl_amd.v2", fromlist=["x"]).build_p2p_transport_plan(
+                          comm_mode="push", copy_elems=1024))
+    try:
+        op = ops[0]
+        assert op.plan.n_groups == 4 and op.plan.row_ends()[-1] == M
+        A_cpu, B_cpu = seeded((M, K), 0, torch.bfloat16), seeded((K, N), 1, torch.bfloat16, scale=K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        blocks = fill_peer_blocks(ops, M, N, torch.bfloat16)
+        op.out.zero_()
+        op.mark_peers_ready()
+        op(A, B, variant)
+        op.check_faults()
+        mine = op.out[:M].clone()
+        assert_gemm_close(mine, A_cpu.float() @ B_cpu.float(), tight=0.032)
+        for p in (1, 2, 3):
+            assert torch.equal(bits(op.peer_out(p)[:M]), bits(mine)), f"push to {p}"
+            assert torch.equal(bits(op.out[p * M:(p + 1) * M]).cpu(), bits(blocks[p])), f"pull from {p}"
+        if variant == "s2":
+            assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts())
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+@pytest.mark.parametrize("local_M,block_m", [(4096, 128), (8192, 128), (8192, 256)])
+def test_baseline_configs_1_and_2_properties(lib, local_M, block_m):
+    """Configs 1 and 2 at full size: all variants give the same bytes, both slices end up
+    identical, the gathered output equals [GEMM rows | peer rows], counters hit tile counts."""
+    M, N, K = local_M, 4096, 1024
+    heaps, ops = make(2, M, N, heap_bytes=1 << 30, block_m=block_m)
+    try:
+        op = ops[0]
+        n_groups = M // (8 * block_m)
+        assert op.plan.n_groups == n_groups and op.plan.tile_counts() == [256] * n_groups
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=K**-0.5))
+        peer = seeded((M, N), 2)
+        results = {}
+        for variant in VARIANTS:
+            op.out.zero_()
+            ops[1].out.zero_()
+            ops[1].out[M:].copy_(peer)
+            op.mark_peers_ready()
+            op(A, B, variant)
+            op.check_faults()
+            assert torch.equal(bits(op.out), bits(op.peer_out(1))), variant  # checksum of checksums: whole slices agree
+            assert torch.equal(bits(op.out[M:]).cpu(), bits(peer)), variant
+            results[variant] = op.out[:M].clone()
+            # idempotence: a second launch changes nothing
+            op.mark_peers_ready()
+            op(A, B, variant)
+            op.check_faults()
+            assert torch.equal(bits(op.out[:M]), bits(results[variant]))
+        assert torch.equal(bits(results["s0"]), bits(results["s1"])) and torch.equal(bits(results["s0"]), bits(results["s2"]))
+        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+        # GEMM numerics on a slab (the CPU matmul of the whole thing is the slow part)
+        rows = slice(M - 256, M)
+        assert_gemm_close(results["s2"][rows], A[rows].float().cpu() @ B.float().cpu(), tight=0.004)
+        # linearity property of the GEMM part: alpha = 2 doubles every output exactly (power of two)
+        op(A, B, "s2", alpha=2.0)
+        op.check_faults()
+        assert torch.equal(op.out[:M].float(), 2 * results["s2"].float())
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+def test_single_rank_is_a_plain_gemm(lib):
+    heaps, ops = make(1, 256, 256)
+    try:
+        A, B = into_heap(heaps[0], seeded((256, 64), 0)), into_heap(heaps[0], seeded((64, 256), 1, scale=1 / 8))
+        for variant in VARIANTS:
+            ops[0].out.zero_()
+            ops[0](A, B, variant)
+            ops[0].check_faults()
+            assert_gemm_close(ops[0].out, A.float().cpu() @ B.float().cpu(), tight=0.004)
+    finally:
+        heaps[0].cleanup()
+
+
+def test_argument_errors(lib):
+    from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(16 << 20, 2)
+    try:
+        op = FusedGemmAllGather(heaps[0], 256, 256)
+        A, B = into_heap(heaps[0], seeded((256, 64), 0)), into_heap(heaps[0], seeded((64, 256), 1))
+        with pytest.raises(ValueError, match="unknown variant 's9'"):
+            op(A, B, "s9")
+        with pytest.raises(ValueError, match=r"C shape mismatch"):
+            op(A[:128], B, "s0")
+        with pytest.raises(ValueError, match="unknown directions='sideways'"):
+            FusedGemmAllGather(heaps[0], 256, 256, directions="sideways")
+    finally:
+        for h in heaps:
+            h.cleanup()

@@ -1,0 +1,112 @@
+"""The MFMA GEMM through the C ABI against the CPU oracle (fp32 matmul, one rounding).
+
+Tolerance: the reference's own (rtol 1e-2, atol 1e-1; tests/test_gemm_allscatter_smoke.py:39-40)
+plus a tight absolute bound that a wrong operand layout or a dropped K step cannot meet."""
+
+import ctypes as C
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import assert_gemm_close, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gemm(lib, A_cpu, B_cpu, out_dtype, **kw):
+    from tileccl_amd import _launch, _lib
+
+    A, B = A_cpu.cuda(), B_cpu.cuda()
+    out = torch.full((A.shape[0], B.shape[1]), float("nan"), dtype=out_dtype, device="cuda")
+    desc = _launch.gemm_desc(A, B, out, **kw)
+    _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
+    torch.cuda.synchronize()
+    return out
+
+
+SHAPES = [
+    (128, 128, 64),  # the reference smoke test's single tile, one K step
+    (128, 64, 128),  # reference smoke shape (M, K, N) = (128, 64, 128)
+    (256, 384, 512),
+    (200, 136, 72),  # ragged M, N and a K tail
+    (1, 8, 8),
+    (130, 8, 264),
+    (512, 512, 256),  # BASELINE config 0
+    (1024, 4096, 1024),
+]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_matches_fp32_matmul(lib, M, N, K, dtype):
+    A = seeded((M, K), 0, dtype)
+    B = seeded((K, N), 1, dtype, scale=K**-0.5)
+    got = run_gemm(lib, A, B, dtype)
+    ref32 = A.float() @ B.float()
+    assert not torch.isnan(got.float()).any()
+    # one rounding of an O(1) value: half an ulp of fp16 (2^-11 rel.) / bf16 (2^-8 rel.) at |x| < 8
+    assert_gemm_close(got, ref32, tight=0.004 if dtype == torch.float16 else 0.032)
+    # the oracle rounds the same fp32 sum once; accumulation order may differ by an fp32 ulp,
+    # which can flip a rounding, so allow one output ulp against it
+    want = oracle.gemm(A, B, dtype)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= (0.004 if dtype == torch.float16 else 0.032)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fp32_output_keeps_the_accumulator(lib, dtype):
+    A, B = seeded((384, 256), 3, dtype), seeded((256, 640), 4, dtype, scale=1 / 16)
+    got = run_gemm(lib, A, B, torch.float32)
+    ref32 = A.float() @ B.float()
+    assert (got.cpu() - ref32).abs().max().item() < 1e-4  # only the fp32 summation order differs
+
+
+def test_alpha_and_plan_tile_256(lib):
+    A, B = seeded((512, 128), 5), seeded((128, 384), 6, scale=128**-0.5)
+    ref32 = 0.5 * (A.float() @ B.float())
+    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5), ref32, tight=0.004)
+    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, group_m=3), ref32, tight=0.004)
+    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, block_n=256, num_wgs=7), ref32, tight=0.004)
+
+
+def test_exact_small_integers(lib):
+    """Integer-valued inputs whose products and sums are exact in fp16/fp32: bit-exact result."""
+    g = torch.Generator().manual_seed(7)
+    A = torch.randint(-3, 4, (256, 192), generator=g).half()
+    B = torch.randint(-3, 4, (192, 256), generator=g).half()
+    got = run_gemm(lib, A, B, torch.float16)
+    assert torch.equal(got.cpu(), (A.float() @ B.float()).half())
+
+
+def test_rows_beyond_M_and_cols_beyond_N_are_untouched(lib):
+    from tileccl_amd import _launch, _lib
+
+    A, B = seeded((100, 64), 8).cuda(), seeded((64, 72), 9).cuda()
+    backing = torch.full((128, 128), 7.0, dtype=torch.float16, device="cuda")
+    out = backing[:100, :72]  # ldc = 128
+    desc = _launch.gemm_desc(A, B, out)
+    _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
+    torch.cuda.synchronize()
+    assert torch.all(backing[100:] == 7.0) and torch.all(backing[:, 72:] == 7.0)
+    assert_gemm_close(out, A.float().cpu() @ B.float().cpu())
+
+
+def test_unsupported_layouts_fail_loudly(lib):
+    from tileccl_amd import _launch, _lib
+
+    A, B = seeded((128, 64), 0).cuda(), seeded((64, 128), 1).cuda()
+    out = torch.empty(128, 128, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError, match="contiguous rows"):
+        _launch.gemm_desc(A, B.t().contiguous().t(), out)
+    with pytest.raises(ValueError, match="K=60 must be a multiple of 8"):
+        d = _launch.gemm_desc(A[:, :60].contiguous(), B[:60].contiguous(), out)
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="N=100 must be a multiple of 8"):
+        d = _launch.gemm_desc(A, B[:, :100].contiguous(), out[:, :100].contiguous())
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="must be a multiple of 128x128"):
+        d = _launch.gemm_desc(A, B, out, block_m=64)
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="no kernel for in_dtype"):
+        d = _launch.gemm_desc(A, B, torch.empty(128, 128, dtype=torch.bfloat16, device="cuda"))
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")

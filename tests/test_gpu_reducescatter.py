@@ -1,0 +1,147 @@
+"""GEMM to ReduceScatter (Gate 2) in the S0 / S1 / S2 variants against the CPU oracle.
+
+The reduction is an fp32 sum of per-rank partials rounded once; with two ranks the sum of
+two fp32 numbers does not depend on order, so the result is bit-exact against the oracle
+run on the partial the GPU produced."""
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import assert_gemm_close, bits, into_heap, seeded
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = ["s0", "s1", "s2"]
+
+
+def make(world, M, N, heap_bytes=256 << 20, **kw):
+    from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(heap_bytes, world)
+    return heaps, [FusedGemmReduceScatter(h, M, N, **kw) for h in heaps]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("partial_dtype,out_dtype", [(torch.float32, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                                    (torch.float32, torch.bfloat16)])
+def test_small_two_ranks_bit_exact(lib, variant, partial_dtype, out_dtype):
+    M, N, K = 512, 512, 256
+    in_dtype = torch.bfloat16 if partial_dtype == torch.bfloat16 else torch.float16
+    heaps, ops = make(2, M, N, partial_dtype=partial_dtype, out_dtype=out_dtype)
+    try:
+        op = ops[0]
+        assert op.plan.groups == [(0, 256, 8), (256, 512, 8)]  # one wave, cut at the owner border
+        A_cpu, B_cpu = seeded((M, K), 0, in_dtype), seeded((K, N), 1, in_dtype, scale=K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        peer = seeded((M, N), 2, partial_dtype)
+        ops[1].partial.copy_(peer)
+        for o in ops:
+            o.out.zero_()
+        op.mark_peers_ready()
+        op(A, B, variant)
+        op.check_faults()
+        assert_gemm_close(op.partial, A_cpu.float() @ B_cpu.float(), tight=1e-4 if partial_dtype == torch.float32 else 0.032)
+        partials = [op.partial.cpu(), peer]
+        for owner in (0, 1):
+            want = oracle.reduce_rows(partials, owner, out_dtype)
+            assert torch.equal(bits(ops[owner].out).cpu(), bits(want)), f"owner {owner}"
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_without_peer_emulation_only_the_own_shard_is_written(lib, variant):
+    M, N, K = 512, 256, 64
+    heaps, ops = make(2, M, N, emulate_peer=False)
+    try:
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=1 / 8))
+        peer = seeded((M, N), 2, torch.float32)
+        ops[1].partial.copy_(peer)
+        for o in ops:
+            o.out.fill_(7.0)
+        ops[0].mark_peers_ready()
+        ops[0](A, B, variant)
+        ops[0].check_faults()
+        want = oracle.reduce_rows([ops[0].partial.cpu(), peer], 0, torch.float16)
+        assert torch.equal(bits(ops[0].out).cpu(), bits(want))
+        assert torch.all(ops[1].out == 7.0)
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_three_ranks_sum_order_owner_first(lib, variant):
+    """With three addends the fp32 sum depends on order: owner first, then ascending ranks."""
+    M, N, K = 768, 264, 64
+    heaps, ops = make(3, M, N, tau_min_bytes=1, group_m=1)
+    try:
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=1 / 8))
+        peers = {p: seeded((M, N), 10 + p, torch.float32) * 1000.0 for p in (1, 2)}  # large magnitudes: order matters
+        for p in (1, 2):
+            ops[p].partial.copy_(peers[p])
+        for o in ops:
+            o.out.zero_()
+        ops[0].mark_peers_ready()
+        ops[0](A, B, variant)
+        ops[0].check_faults()
+        partials = [ops[0].partial.cpu(), peers[1], peers[2]]
+        for owner in range(3):
+            assert torch.equal(bits(ops[owner].out).cpu(), bits(oracle.reduce_rows(partials, owner, torch.float16))), owner
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+def test_baseline_config_3_properties(lib):
+    """8192x2048 @ 2048x4096 fp16, peer partial fp32 N(0,1): variants agree byte for byte,
+    the result equals the oracle on a slab, counters match the plan."""
+    M, N, K = 8192, 4096, 2048
+    heaps, ops = make(2, M, N, heap_bytes=1 << 30)
+    try:
+        op = ops[0]
+        assert op.plan.n_groups == 8 and op.shard_rows == 4096
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=K**-0.5))
+        g = torch.Generator(device="cuda").manual_seed(2)
+        ops[1].partial.normal_(generator=g)
+        outs = {}
+        for variant in VARIANTS:
+            for o in ops:
+                o.out.zero_()
+            op.mark_peers_ready()
+            op(A, B, variant)
+            op.check_faults()
+            outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
+        for v in ("s1", "s2"):
+            assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
+        for owner in (0, 1):
+            rows = slice(owner * 4096, owner * 4096 + 128)
+            want = (op.partial[rows].float() + ops[1].partial[rows].float()).half()
+            assert torch.equal(bits(outs["s2"][owner][:128]), bits(want))
+        rows = slice(4000, 4128)
+        assert_gemm_close(op.partial[rows], A[rows].float().cpu() @ B.float().cpu(), tight=1e-3)
+        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+def test_argument_errors(lib):
+    from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(64 << 20, 3)
+    try:
+        with pytest.raises(ValueError, match=r"M=512 must be divisible by world_size=3"):
+            FusedGemmReduceScatter(heaps[0], 512, 256)
+        op = FusedGemmReduceScatter(heaps[0], 384, 256)  # shards of 128 rows: whole tiles
+        A, B = into_heap(heaps[0], seeded((384, 64), 0)), into_heap(heaps[0], seeded((64, 256), 1))
+        op.mark_peers_ready()
+        op(A, B, "s0")
+        bad = FusedGemmReduceScatter(heaps[0], 192, 256)  # shards of 64 rows cut a 128-row tile
+        with pytest.raises(ValueError, match="shards of whole 128-row plan tiles"):
+            bad(A[:192], B, "s2")
+    finally:
+        for h in heaps:
+            h.cleanup()

@@ -76,73 +76,89 @@ struct Xfer {
   int rows, upr;  // units per row
 };
 
-TCCL_D u32x4 ld16(const char* p) { return __builtin_nontemporal_load((const u32x4*)p); }
-TCCL_D void st16(char* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
+// A window onto a slice region for 16-byte buffer accesses with an explicit cache policy.
+// Byte offsets are 32-bit: every rectangle moved here is far smaller than 4 GiB.
+TCCL_D __amdgpu_buffer_rsrc_t window(int64_t address) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)(uintptr_t)address, 0, 0xffffffffu, 0x00020000);
+}
+template <int kPolicy>
+TCCL_D u32x4 ld16(__amdgpu_buffer_rsrc_t w, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(w, off, 0, kPolicy); }
+template <int kPolicy>
+TCCL_D void st16(__amdgpu_buffer_rsrc_t w, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, w, off, 0, kPolicy); }
 
 constexpr int kThreadsComm = 256;  // threads of a communication workgroup
 constexpr int kCommUnroll = 8;     // 16-byte accesses a thread keeps in flight
 
 // ---- copy: units [u_lo, u_hi) of the rectangle, one source slice, any number of targets ----
+// kPolicy is the cache policy of both sides: kCoherent inside fused launches (the source
+// was just written by other workgroups, the target will be read by a peer), kStreaming
+// for the stand-alone bulk kernel.
+template <int kPolicy>
 TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const int tid = threadIdx.x;
   const int src_rank = __builtin_ctz(x.src_ranks);
-  const char* src = (const char*)(uintptr_t)(a.heap_bases[src_rank] + x.src_off);
+  const __amdgpu_buffer_rsrc_t src = window(a.heap_bases[src_rank] + x.src_off);
   const bool flat = (x.src_pitch == (int64_t)x.upr * 16) && (x.dst_pitch == x.src_pitch);
+  const uint32_t sp = (uint32_t)x.src_pitch, dp = (uint32_t)x.dst_pitch;
   for (int u0 = u_lo; u0 < u_hi; u0 += kThreadsComm * kCommUnroll) {
     u32x4 v[kCommUnroll];
-    int64_t doff[kCommUnroll];
+    uint32_t doff[kCommUnroll];
 #pragma unroll
     for (int k = 0; k < kCommUnroll; ++k) {
       const int u = u0 + tid + k * kThreadsComm;
-      if (u < u_hi) {
-        int64_t soff;
-        if (flat) {
-          soff = (int64_t)u * 16;
-          doff[k] = soff;
-        } else {
-          const int r = u / x.upr, c = u - r * x.upr;
-          soff = r * x.src_pitch + (int64_t)c * 16;
-          doff[k] = r * x.dst_pitch + (int64_t)c * 16;
-        }
-        v[k] = ld16(src + soff);
+      uint32_t soff;
+      if (flat) {
+        soff = (uint32_t)u * 16u;
+        doff[k] = soff;
+      } else {
+        const uint32_t r = (uint32_t)u / (uint32_t)x.upr, c = (uint32_t)u - r * (uint32_t)x.upr;
+        soff = r * sp + c * 16u;
+        doff[k] = r * dp + c * 16u;
       }
+      if (u >= u_hi) soff = 0;  // idle lane: harmless re-read of the first unit, nothing stored
+      v[k] = ld16<kPolicy>(src, soff);
     }
     for (int q = 0; q < a.world; ++q) {
       if (!((x.dst_ranks >> q) & 1u)) continue;
-      char* dst = (char*)(uintptr_t)(a.heap_bases[q] + x.dst_off);
+      const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[q] + x.dst_off);
 #pragma unroll
-      for (int k = 0; k < kCommUnroll; ++k) {
-        const int u = u0 + tid + k * kThreadsComm;
-        if (u < u_hi) st16(dst + doff[k], v[k]);
-      }
+      for (int k = 0; k < kCommUnroll; ++k)
+        if (u0 + tid + k * kThreadsComm < u_hi) st16<kPolicy>(dst, doff[k], v[k]);
     }
   }
 }
 
 // ---- reduce: 8 elements per unit, fp32 accumulation, one rounding to the output type --------
-template <typename PT>
-TCCL_D void load8(const char* p, float (&f)[8]);
-template <>
-TCCL_D void load8<float>(const char* p, float (&f)[8]) {
-  const u32x4 a = ld16(p), b = ld16(p + 16);
+template <typename PT, int kPolicy>
+struct Load8;
+template <int kPolicy>
+struct Load8<float, kPolicy> {
+  static TCCL_D void run(__amdgpu_buffer_rsrc_t w, uint32_t off, float (&f)[8]) {
+    const f32x4v a = __builtin_bit_cast(f32x4v, ld16<kPolicy>(w, off));
+    const f32x4v b = __builtin_bit_cast(f32x4v, ld16<kPolicy>(w, off + 16));
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    f[e] = __builtin_bit_cast(float, a[e]);
-    f[4 + e] = __builtin_bit_cast(float, b[e]);
+    for (int e = 0; e < 4; ++e) {
+      f[e] = a[e];
+      f[4 + e] = b[e];
+    }
   }
-}
-template <>
-TCCL_D void load8<_Float16>(const char* p, float (&f)[8]) {
-  const f16x8v h = __builtin_bit_cast(f16x8v, ld16(p));
+};
+template <int kPolicy>
+struct Load8<_Float16, kPolicy> {
+  static TCCL_D void run(__amdgpu_buffer_rsrc_t w, uint32_t off, float (&f)[8]) {
+    const f16x8v h = __builtin_bit_cast(f16x8v, ld16<kPolicy>(w, off));
 #pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
-}
-template <>
-TCCL_D void load8<__bf16>(const char* p, float (&f)[8]) {
-  const bf16x8v h = __builtin_bit_cast(bf16x8v, ld16(p));
+    for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
+  }
+};
+template <int kPolicy>
+struct Load8<__bf16, kPolicy> {
+  static TCCL_D void run(__amdgpu_buffer_rsrc_t w, uint32_t off, float (&f)[8]) {
+    const bf16x8v h = __builtin_bit_cast(bf16x8v, ld16<kPolicy>(w, off));
 #pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
-}
+    for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
+  }
+};
 
 template <typename OT>
 TCCL_D u32x4 pack8(const float (&f)[8]);
@@ -161,49 +177,74 @@ TCCL_D u32x4 pack8<__bf16>(const float (&f)[8]) {
   return __builtin_bit_cast(u32x4, h);
 }
 
+constexpr int kReduceUnroll = 2;
+
 // Sum order: the owner's addend first, then the other ranks in ascending order
 // (tile_reduce_scatter: local chunk, then peers ascending; collectives.py:766-781).
-template <typename PT, typename OT>
+template <typename PT, typename OT, int kPolicy>
 TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
-  constexpr int kSrcUnit = 8 * sizeof(PT);
+  constexpr uint32_t kSrcUnit = 8 * sizeof(PT);
   const int tid = threadIdx.x;
   const int dst_rank = __builtin_ctz(x.dst_ranks);
-  char* dst = (char*)(uintptr_t)(a.heap_bases[dst_rank] + x.dst_off);
-  const char* first = (const char*)(uintptr_t)(a.heap_bases[x.first_rank] + x.src_off);
-  for (int u = u_lo + tid; u < u_hi; u += kThreadsComm) {
-    const int r = u / x.upr, c = u - r * x.upr;
-    const int64_t soff = r * x.src_pitch + (int64_t)c * kSrcUnit;
-    float acc[8];
-    load8<PT>(first + soff, acc);
+  const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[dst_rank] + x.dst_off);
+  const __amdgpu_buffer_rsrc_t first = window(a.heap_bases[x.first_rank] + x.src_off);
+  const uint32_t sp = (uint32_t)x.src_pitch, dp = (uint32_t)x.dst_pitch;
+  for (int u0 = u_lo; u0 < u_hi; u0 += kThreadsComm * kReduceUnroll) {
+    float acc[kReduceUnroll][8];
+    uint32_t soff[kReduceUnroll], doff[kReduceUnroll];
+#pragma unroll
+    for (int k = 0; k < kReduceUnroll; ++k) {
+      const int u = u0 + tid + k * kThreadsComm;
+      const uint32_t r = (uint32_t)u / (uint32_t)x.upr, c = (uint32_t)u - r * (uint32_t)x.upr;
+      soff[k] = r * sp + c * kSrcUnit;
+      doff[k] = r * dp + c * 16u;
+      if (u >= u_hi) soff[k] = 0;  // idle lane: harmless re-read, nothing stored
+      Load8<PT, kPolicy>::run(first, soff[k], acc[k]);
+    }
     for (int p = 0; p < a.world; ++p) {
       if (p == x.first_rank || !((x.src_ranks >> p) & 1u)) continue;
-      float in[8];
-      load8<PT>((const char*)(uintptr_t)(a.heap_bases[p] + x.src_off) + soff, in);
+      const __amdgpu_buffer_rsrc_t other = window(a.heap_bases[p] + x.src_off);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += in[e];
+      for (int k = 0; k < kReduceUnroll; ++k) {
+        float in[8];
+        Load8<PT, kPolicy>::run(other, soff[k], in);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[k][e] += in[e];
+      }
     }
-    st16(dst + r * x.dst_pitch + (int64_t)c * 16, pack8<OT>(acc));
+#pragma unroll
+    for (int k = 0; k < kReduceUnroll; ++k)
+      if (u0 + tid + k * kThreadsComm < u_hi) st16<kPolicy>(dst, doff[k], pack8<OT>(acc[k]));
   }
 }
 
+template <int kPolicy>
 TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const int key = a.partial_dtype * 4 + a.out_dtype;
   switch (key) {
-    case kF32 * 4 + kF16: run_reduce_t<float, _Float16>(a, x, u_lo, u_hi); break;
-    case kF32 * 4 + kBF16: run_reduce_t<float, __bf16>(a, x, u_lo, u_hi); break;
-    case kF16 * 4 + kF16: run_reduce_t<_Float16, _Float16>(a, x, u_lo, u_hi); break;
-    case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16>(a, x, u_lo, u_hi); break;
-    case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16>(a, x, u_lo, u_hi); break;
-    case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kF16: run_reduce_t<float, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kBF16: run_reduce_t<float, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kF16: run_reduce_t<_Float16, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
     default: break;
   }
 }
 
 TCCL_D void run_xfer(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
-  if (x.reduce)
-    run_reduce(a, x, u_lo, u_hi);
-  else
-    run_copy(a, x, u_lo, u_hi);
+  const bool fused = a.granularity != kBulk;
+  if (x.reduce) {
+    if (fused)
+      run_reduce<kCoherent>(a, x, u_lo, u_hi);
+    else
+      run_reduce<kStreaming>(a, x, u_lo, u_hi);
+  } else {
+    if (fused)
+      run_copy<kCoherent>(a, x, u_lo, u_hi);
+    else
+      run_copy<kStreaming>(a, x, u_lo, u_hi);
+  }
 }
 
 // ---- rectangles of the three operations ----------------------------------------------------------
@@ -282,8 +323,7 @@ struct Waiter {
     __syncthreads();
     const bool all_ok = *verdict != 0;
     __syncthreads();
-    observe_fence();
-    return all_ok;
+    return all_ok;  // the data itself is read with device-coherent loads: no cache invalidate
   }
 
   // S1: locks[tile] of `rank`'s slice.  Own locks are consumed (tile_wait); a peer's are
@@ -292,7 +332,7 @@ struct Waiter {
     bool ok = true;
     if (threadIdx.x == 0) {
       int32_t* w = translate_ptr(a.locks, a.rank, rank, a.heap_bases);
-      ok = tile_wait(w, tile_id, /*consume=*/rank == a.rank, deadline);
+      ok = tile_wait<true>(w, tile_id, /*consume=*/rank == a.rank, deadline);
     }
     return finish(ok);
   }
@@ -303,7 +343,7 @@ struct Waiter {
     if (threadIdx.x == 0) {
       const int32_t need = a.epoch * a.tile_counts[g];
       for (int r = 0; r < a.world && ok; ++r)
-        if ((ranks >> r) & 1u) ok = tile_wait_ge(translate_ptr(a.counter, a.rank, r, a.heap_bases), g, need, deadline);
+        if ((ranks >> r) & 1u) ok = tile_wait_ge<true>(translate_ptr(a.counter, a.rank, r, a.heap_bases), g, need, deadline);
       if (ok && a.trace_ready_clock) {
         unsigned long long* slot = (unsigned long long*)&a.trace_ready_clock[g];
         atomicCAS(slot, 0ull, (unsigned long long)now_ticks());
@@ -315,12 +355,12 @@ struct Waiter {
 
 // A finished task of group g: count it; the task that completes the group stamps the clock.
 TCCL_D void task_done(const CommArgs& a, int g, int tasks_of_group) {
-  publish_fence();
+  wait_vmem();  // this wave's write-through stores have landed
   __syncthreads();
   if (threadIdx.x == 0) {
     if (a.trace_comm_counter) atomicAdd(&a.trace_comm_counter[g], 1);
     if (a.barrier) {
-      const int32_t prev = tile_signal_add(a.barrier, g, 1);
+      const int32_t prev = tile_signal_add<true>(a.barrier, g, 1);
       if (prev + 1 == a.epoch * tasks_of_group && a.trace_done_clock) a.trace_done_clock[g] = now_ticks();
     }
   }

@@ -70,22 +70,42 @@ TCCL_D T* translate_ptr(T* ptr, int from_rank, int to_rank, const int64_t* heap_
 TCCL_D int64_t now_ticks() { return (int64_t)wall_clock64(); }
 
 // ---------------------------------------------------------------------------------------
-// Signal words (int32, in the heap).  One GPU: agent scope is enough for every
-// workgroup on every XCD to observe a release; real peers would need system scope
-// (the reference's v1 default is "gpu", v2 "sys": sync/primitives.py:357, ipc.py:137).
+// Signal words (int32, in the heap).
+//
+// Two flavours of every primitive:
+//  * the stand-alone form carries the ordering itself (release on signal, acquire on a
+//    successful wait), like the reference's Triton atomics with sem="release"/"acquire"
+//    (sync/primitives.py:357-500, tileccl_v2/ipc.py:137-254);
+//  * the `Relaxed` form is for the fused kernels, whose *data path* is already coherent:
+//    producers store finished output with device-coherent write-through stores
+//    (kCoherent cache policy) and wait for them to complete before signalling, consumers
+//    read with device-coherent loads.  An agent-scope release/acquire on gfx950 writes
+//    back / invalidates the whole per-XCD L2; doing that once per tile from hundreds of
+//    workgroups evicts the GEMM's operands over and over, so the fused path avoids it.
+// One GPU: agent scope reaches every workgroup on every XCD; real peers would need system
+// scope (the reference's v1 default is "gpu", v2 "sys").
 // ---------------------------------------------------------------------------------------
 
-// tile_signal: locks[i] = 1, release.  (sync/primitives.py:357-387)
+// Cache policy bits of raw buffer loads/stores on gfx950: sc0 = 1, nt = 2, sc1 = 16.
+constexpr int kCoherent = 17;  // sc0 sc1: write through to / read from memory, visible to every XCD
+constexpr int kStreaming = 2;  // nt: data is touched once
+
+// All of this wave's outstanding global loads and stores have completed.
+TCCL_D void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <bool Relaxed = false>
 TCCL_D void tile_signal(int32_t* locks, int i) {
-  __hip_atomic_exchange(&locks[i], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_exchange(&locks[i], 1, Relaxed ? __ATOMIC_RELAXED : __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // One CAS probe: consuming (1 -> 0, tile_wait / tile_try_wait) or non-consuming
 // (1 -> 1, tile_poll / tile_try_poll).  (sync/primitives.py:390-439, ipc.py:193-228)
+template <bool Relaxed = false>
 TCCL_D bool tile_probe(int32_t* locks, int i, bool consume) {
   int32_t expected = 1;
-  return __hip_atomic_compare_exchange_strong(&locks[i], &expected, consume ? 0 : 1, __ATOMIC_ACQUIRE,
-                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_compare_exchange_strong(&locks[i], &expected, consume ? 0 : 1,
+                                              Relaxed ? __ATOMIC_RELAXED : __ATOMIC_ACQUIRE, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // tile_try_wait / tile_try_poll: at most max_spins probes; true when the flag was seen.
@@ -97,39 +117,43 @@ TCCL_D bool tile_try_wait(int32_t* locks, int i, int max_spins, bool consume) {
 
 // tile_wait / tile_poll with a deadline: the reference spins forever
 // (sync/primitives.py:390-414); here every wait gives up at `deadline` (now_ticks units)
-// and reports false so the kernel can drain and the host can raise.
+// and reports false so the kernel can drain and the host can raise.  The spin reads the
+// word with relaxed loads; the CAS runs once the flag has been seen.
+template <bool Relaxed = false>
 TCCL_D bool tile_wait(int32_t* locks, int i, bool consume, int64_t deadline) {
   for (;;) {
-    if (tile_try_wait(locks, i, 64, consume)) return true;
-    if (now_ticks() > deadline) return false;
-    __builtin_amdgcn_s_sleep(2);
-  }
-}
-
-// tile_signal_add: counter[i] += v, release; returns the previous value. (ipc.py:231-241)
-TCCL_D int32_t tile_signal_add(int32_t* words, int i, int32_t v) {
-  return __hip_atomic_fetch_add(&words[i], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// tile_wait_ge: spin until counter[i] >= threshold (acquire).  The reference reads the
-// word with atomic_add(0) (ipc.py:244-254); an acquire load observes the same value
-// without taking the line exclusive.  Bounded like tile_wait.
-TCCL_D bool tile_wait_ge(const int32_t* words, int i, int32_t threshold, int64_t deadline) {
-  for (;;) {
     for (int s = 0; s < 32; ++s) {
-      if (__hip_atomic_load(&words[i], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) >= threshold) return true;
-      __builtin_amdgcn_s_sleep(1);
+      if (__hip_atomic_load(&locks[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1) {
+        if (tile_probe<Relaxed>(locks, i, consume)) return true;
+      }
+      __builtin_amdgcn_s_sleep(4);
     }
     if (now_ticks() > deadline) return false;
   }
 }
 
-// Every thread of the workgroup has finished its global stores -> make them visible at
-// agent scope before one thread publishes the signal.
-TCCL_D void publish_fence() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
-// After one thread's acquire-wait and a workgroup barrier, every other thread drops
-// stale cache lines before reading the signalled data.
-TCCL_D void observe_fence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+// tile_signal_add: counter[i] += v; returns the previous value. (ipc.py:231-241)
+template <bool Relaxed = false>
+TCCL_D int32_t tile_signal_add(int32_t* words, int i, int32_t v) {
+  return __hip_atomic_fetch_add(&words[i], v, Relaxed ? __ATOMIC_RELAXED : __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// tile_wait_ge: spin until counter[i] >= threshold.  The reference reads the word with
+// atomic_add(0, acquire) (ipc.py:244-254); relaxed loads followed by one acquire fence
+// observe the same value without taking the line exclusive.  Bounded like tile_wait.
+template <bool Relaxed = false>
+TCCL_D bool tile_wait_ge(const int32_t* words, int i, int32_t threshold, int64_t deadline) {
+  for (;;) {
+    for (int s = 0; s < 32; ++s) {
+      if (__hip_atomic_load(&words[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= threshold) {
+        if (!Relaxed) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        return true;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+    if (now_ticks() > deadline) return false;
+  }
+}
 #endif  // __HIPCC__
 
 }  // namespace tccl

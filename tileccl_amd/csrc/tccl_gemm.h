@@ -197,6 +197,7 @@ struct GemmRole {
   // ---- accumulators -> LDS -> global -------------------------------------------------------
   // Each wave stages its own 32-row slab (one bi at a time) in a private LDS window, then
   // writes it out with 16-byte stores that are contiguous along the row.
+  template <int kPolicy>
   TCCL_D void epilogue(int row0, int col0, const f32x16 (&acc)[2][2]) const {
     constexpr int kEsz = sizeof(OutT);
     constexpr int kRowBytes = 64 * kEsz;       // one wave row: 64 columns
@@ -204,7 +205,11 @@ struct GemmRole {
     constexpr int kPerChunk = 16 / kEsz;       // elements per chunk
     char* win = lds + wave * (32 * 64 * 4);    // 8 KiB window per wave (fp32 worst case)
     const int half = lane >> 5, l32 = lane & 31;
-    OutT* C = (OutT*)g.C;
+    // Stores go through a buffer resource rooted at the sub-tile so that the cache policy
+    // can be chosen: plain write-back when nobody waits for the tile, device-coherent
+    // write-through when a communication workgroup will read it right after the signal.
+    OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
+    const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
 
 #pragma unroll
     for (int bi = 0; bi < 2; ++bi) {
@@ -235,15 +240,16 @@ struct GemmRole {
       for (int r = 0; r < (32 * kChunks) / 64; ++r) {
         const int idx = lane + 64 * r;
         const int row = idx / kChunks, chunk = idx % kChunks;
-        const uint4 v = *(const uint4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
-        const int grow = row0 + wm * 64 + bi * 32 + row;
-        const int gcol = col0 + wn * 64 + chunk * kPerChunk;
-        if (grow < g.M && gcol < g.N) *(uint4*)(C + (int64_t)grow * g.ldc + gcol) = v;
+        const u32x4 v = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
+        const int lrow = wm * 64 + bi * 32 + row, lcol = wn * 64 + chunk * kPerChunk;
+        if (row0 + lrow < g.M && col0 + lcol < g.N)
+          __builtin_amdgcn_raw_buffer_store_b128(v, rc, (uint32_t)((lrow * g.ldc + lcol) * kEsz), 0, kPolicy);
       }
     }
   }
 
   // ---- one 128 x 128 sub-tile -------------------------------------------------------------------
+  template <int kPolicy>
   TCCL_D void subtile(int row0, int col0) const {
     f32x16 acc[2][2];
 #pragma unroll
@@ -265,7 +271,7 @@ struct GemmRole {
       if (kt + 1 < ksteps) load_global(src, kt + 1, ragged && kt + 2 == ksteps, ra, rb);
       compute(acc);
     }
-    epilogue(row0, col0, acc);
+    epilogue<kPolicy>(row0, col0, acc);
   }
 
   // ---- persistent loop over plan tiles ----------------------------------------------------------
@@ -277,16 +283,22 @@ struct GemmRole {
       for (int sm = 0; sm < g.block_m; sm += kTile)
         for (int sn = 0; sn < g.block_n; sn += kTile) {
           const int row0 = tc.m * g.block_m + sm, col0 = tc.n * g.block_n + sn;
-          if (row0 < g.M && col0 < g.N) subtile(row0, col0);
+          if (row0 >= g.M || col0 >= g.N) continue;
+          if (s.mode == kSignalNone)
+            subtile<0>(row0, col0);
+          else
+            subtile<kCoherent>(row0, col0);
         }
       if (s.mode != kSignalNone) {
-        publish_fence();
+        // The tile was stored write-through; once every wave's stores have completed the
+        // data is visible device-wide and one lane may publish the signal.
+        wait_vmem();
         __syncthreads();
         if (tid == 0) {
           if (s.mode == kSignalTile)
-            tile_signal(s.locks, tile_id);
+            tile_signal<true>(s.locks, tile_id);
           else
-            tile_signal_add(s.counter, s.group_table[tile_id], 1);
+            tile_signal_add<true>(s.counter, s.group_table[tile_id], 1);
         }
       }
     }

@@ -135,13 +135,16 @@ class _FusedBase:
             self.heap.peer_view(self.signals.counter, peer).fill_(PEER_READY)
             self.heap.peer_view(self.locks, peer).fill_(1)
 
-    def _descs(self, directions: int):
+    def _descs(self, directions: int, variant: str):
         assert self.words is not None
+        if variant not in _launch.VARIANTS:
+            raise ValueError(f"unknown variant {variant!r}; expected one of {sorted(_launch.VARIANTS)}")
         view = _launch.heap_view(self.heap.get_heap_bases(), self.rank, self.world_size)
         transport = _launch.transport_desc(
             directions, self.transport.copy_elems, self.transport.reduce_elems, self.num_comm_wgs
         )
-        self.words.next_epoch()
+        if variant == "s2":  # only S2 launches add to the counters, so only they advance the epoch
+            self.words.next_epoch()
         return view, transport, self.words.desc()
 
     def check_faults(self) -> None:
@@ -176,7 +179,7 @@ class FusedGemmAllGather(_FusedBase):
             A, B, self.local_block, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
             alpha=alpha, num_wgs=self.num_gemm_wgs,
         )
-        view, transport, sync = self._descs(self.directions)
+        view, transport, sync = self._descs(self.directions, variant)
         rc = _lib.load().tccl_gemm_allgather(
             C.byref(gemm), _launch.ptr(self.out), int(self.out.stride(0)), C.byref(view), C.byref(sync),
             C.byref(transport), _launch.VARIANTS[variant], _launch.stream_ptr(),
@@ -220,7 +223,7 @@ class FusedGemmReduceScatter(_FusedBase):
             A, B, self.partial, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
             alpha=alpha, num_wgs=self.num_gemm_wgs,
         )
-        view, transport, sync = self._descs(_lib.DIR_PULL)
+        view, transport, sync = self._descs(_lib.DIR_PULL, variant)
         rc = _lib.load().tccl_gemm_reducescatter(
             C.byref(gemm), _launch.ptr(self.out), _launch.dtype_code(self.out.dtype), int(self.out.stride(0)),
             C.byref(view), C.byref(sync), C.byref(transport), int(self.emulate_peer),
