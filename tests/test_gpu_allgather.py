@@ -133,10 +133,14 @@ def test_baseline_configs_1_and_2_properties(lib, local_M, block_m):
         # GEMM numerics on a slab (the CPU matmul of the whole thing is the slow part)
         rows = slice(M - 256, M)
         assert_gemm_close(results["s2"][rows], A[rows].float().cpu() @ B.float().cpu(), tight=0.004)
-        # linearity property of the GEMM part: alpha = 2 doubles every output exactly (power of two)
+        # linearity property of the GEMM part: alpha = 2 doubles every normal-range output exactly
+        # (scaling by a power of two commutes with rounding except among fp16 subnormals)
         op(A, B, "s2", alpha=2.0)
         op.check_faults()
-        assert torch.equal(op.out[:M].float(), 2 * results["s2"].float())
+        doubled, base = op.out[:M].float(), results["s2"].float()
+        normal = base.abs() >= 2.0**-13
+        assert torch.equal(doubled[normal], 2 * base[normal])
+        assert (doubled - 2 * base).abs().max().item() <= 2.0**-23
     finally:
         for h in heaps:
             h.cleanup()

@@ -39,7 +39,7 @@ def test_gemm_allscatter_single_gpu_smoke(lib):
             heap.cleanup()
 
 
-def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, **pattern_kw):
+def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, inspect=None, **pattern_kw):
     import tileccl_amd as tileccl
     from tileccl_amd import ops
 
@@ -74,7 +74,8 @@ def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, **pattern_kw)
         # Same inputs on every rank -> every rank's local GEMM is bit-identical, so all C agree bit for bit.
         for r in range(1, world):
             assert torch.equal(bits(Cs[0]), bits(Cs[r]))
-        return plans
+        if inspect is not None:
+            inspect(plans)  # while the heaps (and the signal words in them) are still alive
     finally:
         for c in ctxs:
             c.heap.cleanup()
@@ -83,10 +84,12 @@ def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, **pattern_kw)
 @pytest.mark.parametrize("pattern", PATTERNS)
 def test_baseline_config_0(lib, pattern):
     """512x256 @ 256x512 fp16, seed 0, world 2, tiles 128x128: each slice ends with the full C."""
-    plans = _two_rank_case(pattern, 512, 256, 512)
-    if pattern == "tile_group":
-        plan = plans[0].pattern_impl.last_plan
-        assert plan.groups == [(0, 512, 16)] and plan.group_table.tolist() == [0] * 16
+    def inspect(plans):
+        if pattern == "tile_group":
+            plan = plans[0].pattern_impl.last_plan
+            assert plan.groups == [(0, 512, 16)] and plan.group_table.tolist() == [0] * 16
+
+    _two_rank_case(pattern, 512, 256, 512, inspect=inspect)
 
 
 @pytest.mark.parametrize("pattern", PATTERNS)
@@ -95,13 +98,15 @@ def test_ragged_rows_three_ranks_bf16(lib, pattern):
 
 
 def test_tile_group_counters_and_many_groups(lib):
-    plans = _two_rank_case("tile_group", 2048, 64, 256, tau_min_bytes=1, GROUP_M=2)
-    impl = plans[0].pattern_impl
-    plan, words = impl.last_plan, impl._last_sync
-    assert plan.n_groups == 8 and plan.tile_counts() == [4] * 8
-    assert words.counter.tolist() == oracle.expected_counters(plan.tile_counts(), words.epoch)
-    # each group: cols/.. one push task per group (2048*128 elems / 16384 = 16 per 256 rows)
-    assert all(b > 0 for b in words.barrier.tolist())
+    def inspect(plans):
+        impl = plans[0].pattern_impl
+        plan, words = impl.last_plan, impl._last_sync
+        assert plan.n_groups == 8 and plan.tile_counts() == [4] * 8
+        assert words.counter.tolist() == oracle.expected_counters(plan.tile_counts(), words.epoch)
+        # a group's column block is 256 rows x 128 cols = 32768 elements = 2 push tasks of 16384
+        assert words.barrier.tolist() == [2] * 8
+
+    _two_rank_case("tile_group", 2048, 64, 256, tau_min_bytes=1, GROUP_M=2, inspect=inspect)
 
 
 def test_repeated_launches_reuse_unreset_counters(lib):
