@@ -1,0 +1,103 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol the header declares,
+rejects bad descriptors before touching a device, and its host-side index helpers (the very
+functions the kernels inline) agree with the loop-form oracle."""
+
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+from oracle import planning as ref
+
+HEADER = Path(__file__).resolve().parent.parent / "include" / "tileccl_hip.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(tccl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_typed(lib):
+    from tileccl_amd import _lib
+
+    names = declared_functions()
+    assert len(names) >= 19 and "tccl_gemm_allgather" in names
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names  # the ctypes table covers the header exactly
+    assert lib.tccl_abi_version() == 1
+
+
+def test_struct_layouts_match_the_header():
+    from tileccl_amd import _lib
+
+    # sizes follow from the header's field lists under the natural C alignment rules
+    assert C.sizeof(_lib.GemmDesc) == 3 * 8 + 3 * 4 + 4 + 3 * 8 + 2 * 4 + 4 + 3 * 4 + 4 + 3 * 4
+    assert C.sizeof(_lib.HeapView) == 16 and C.sizeof(_lib.ScatterDesc) == 16 and C.sizeof(_lib.TransportDesc) == 16
+    assert C.sizeof(_lib.SyncDesc) == 4 * 8 + 2 * 4 + 8 * 8 + 8
+    assert C.sizeof(_lib.DeviceInfo) == 8 * 4 + 64
+    assert _lib.GemmDesc.lda.offset == 40 and _lib.SyncDesc.row_starts.offset == 40
+
+
+def test_bad_descriptors_are_rejected_on_the_host(lib):
+    from tileccl_amd import _lib
+
+    assert lib.tccl_gemm(None, None) == _lib.ERR_INVALID
+    assert b"NULL" in lib.tccl_last_error_string()
+    d = _lib.GemmDesc()
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_INVALID
+    d.A = d.B = d.C = 0x1000
+    d.M, d.N, d.K = 128, 128, 0
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_INVALID
+    assert b"M, N, K must be positive" in lib.tccl_last_error_string()
+    d.K = 64
+    d.lda, d.ldb, d.ldc = 64, 128, 128
+    d.block_m, d.block_n, d.group_m = 96, 128, 8
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_UNSUPPORTED
+    d.block_m = 128
+    d.in_dtype = _lib.F32
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_UNSUPPORTED
+    d.in_dtype = _lib.F16
+    d.A = 0x1008  # not 16-byte aligned
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_UNSUPPORTED
+    with pytest.raises(ValueError, match="16-byte boundaries"):
+        _lib.check(_lib.ERR_UNSUPPORTED, "tccl_gemm")
+    with pytest.raises(RuntimeError, match="HIP error in x: error code 2"):
+        _lib.check(2, "x")
+    h = _lib.HeapView(0x1000, 3, 2)
+    assert lib.tccl_exchange_rows(0x1000, 8, 8, 8, 2, C.byref(h), None, None) == _lib.ERR_INVALID
+    assert b"rank=3 out of range for world_size=2" in lib.tccl_last_error_string()
+    assert lib.tccl_heap_create(0, 2, None, None) == _lib.ERR_INVALID
+    assert lib.tccl_heap_destroy(None) == 0
+    assert lib.tccl_fill_i32(None, 0, 0, None) == 0
+
+
+@pytest.mark.parametrize("tile_rows,tile_cols,group_m", [(32, 32, 8), (12, 2, 8), (7, 5, 3), (1, 9, 8), (64, 32, 8), (5, 1, 1)])
+def test_device_tile_order_equals_the_reference_swizzle(lib, tile_rows, tile_cols, group_m):
+    tm, tn = C.c_int32(), C.c_int32()
+    seen = set()
+    for t in range(tile_rows * tile_cols):
+        assert lib.tccl_tile_coords(t, tile_rows, tile_cols, group_m, C.byref(tm), C.byref(tn)) == 0
+        assert (tm.value, tn.value) == ref.swizzle(t, tile_rows, tile_cols, group_m)
+        seen.add((tm.value, tn.value))
+    assert len(seen) == tile_rows * tile_cols  # a bijection onto the tile grid
+    assert lib.tccl_tile_coords(tile_rows * tile_cols, tile_rows, tile_cols, group_m, C.byref(tm), C.byref(tn)) != 0
+
+
+@pytest.mark.parametrize("total,xcds,span", [(1024, 8, 32), (1000, 8, 32), (16, 8, 8), (2048, 8, 32), (513, 8, 4), (64, 1, 1), (4096, 8, 64)])
+def test_xcd_remap_is_a_bijection_and_keeps_blocks(lib, total, xcds, span):
+    out = C.c_int32()
+    ids = []
+    for slot in range(total):
+        assert lib.tccl_tile_for_slot(slot, total, xcds, span, C.byref(out)) == 0
+        ids.append(out.value)
+    assert sorted(ids) == list(range(total))
+    block = xcds * span
+    for slot, tile in enumerate(ids):
+        assert slot // block == tile // block  # a slot never leaves its block of xcds*span ids
+        if xcds > 1 and (slot // block + 1) * block <= total:
+            # XCD slot % xcds takes the span ids [x*span, (x+1)*span) of the block, in order
+            assert (tile % block) // span == slot % xcds and (tile % block) % span == (slot % block) // xcds
+        else:
+            assert tile == slot

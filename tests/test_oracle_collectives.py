@@ -1,0 +1,100 @@
+"""Pins for the collective half of the oracle: the vectorised placement against an
+element-by-element loop with the reference's mask, exactness of the reduce, the gather
+layout, and the GEMM restatement against hand-computable cases."""
+
+import pytest
+import torch
+
+from oracle import collectives as oc
+from tileccl_amd.patterns.contracts import resolve_pattern_execution
+
+
+def test_gemm_restatement_on_hand_computable_inputs():
+    A = torch.tensor([[1.0, 2.0], [3.0, 4.0]], dtype=torch.float16)
+    B = torch.tensor([[5.0, 6.0], [7.0, 8.0]], dtype=torch.float16)
+    assert oc.gemm(A, B, torch.float16).tolist() == [[19.0, 22.0], [43.0, 50.0]]
+    assert oc.gemm(A, B, torch.float32, alpha=0.5).tolist() == [[9.5, 11.0], [21.5, 25.0]]
+    # fp32 accumulation, one rounding: 2049 = 2048 + 1 is not an fp16 number and rounds to even (2048)
+    ones = torch.ones(1, 2049, dtype=torch.float16)
+    assert oc.gemm(ones, ones.t().contiguous(), torch.float16).item() == 2048.0
+    assert oc.gemm(ones, ones.t().contiguous(), torch.float32).item() == 2049.0
+    # identity
+    g = torch.Generator().manual_seed(0)
+    X = torch.randn(16, 16, generator=g).half()
+    assert torch.equal(oc.gemm(X, torch.eye(16, dtype=torch.float16), torch.float16), X)
+
+
+@pytest.mark.parametrize("M,N,world,rank", [(200, 264, 3, 1), (256, 256, 2, 0), (130, 48, 2, 1), (128, 512, 4, 3)])
+def test_vectorised_placement_equals_the_masked_tile_loop(M, N, world, rank):
+    g = torch.Generator().manual_seed(M + N)
+    local = torch.randn(M, N, generator=g).half()
+    spec = resolve_pattern_execution(torch.empty(M, 8), torch.empty(8, N), local, rank=rank, world_size=world,
+                                     b_layout="full", c_layout="full")
+    args = (spec.scatter_src_col_offset, spec.scatter_cols, spec.scatter_dst_leading_dim, spec.scatter_dst_col_offset)
+    fast, slow = torch.zeros(M, N, dtype=torch.float16), torch.zeros(M, N, dtype=torch.float16)
+    oc.scatter_into_peer(fast, local, *args)
+    oc.scatter_into_peer_by_tiles(slow, local, *args, block_m=64, block_n=64)
+    assert torch.equal(fast, slow)
+    shard = N // world
+    assert torch.equal(fast[:, rank * shard:(rank + 1) * shard], local[:, rank * shard:(rank + 1) * shard])
+    mask = torch.ones(N, dtype=torch.bool)
+    mask[rank * shard:(rank + 1) * shard] = False
+    assert torch.count_nonzero(fast[:, mask]).item() == 0  # nothing outside the rank's block is touched
+
+
+def test_shard_layout_placement_uses_its_own_leading_dimension():
+    local = torch.arange(12, dtype=torch.float16).reshape(3, 4)
+    dest = torch.zeros(3, 4, dtype=torch.float16)
+    oc.scatter_into_peer(dest, local, 0, 4, 4, 0)
+    assert torch.equal(dest, local)
+    wide = torch.zeros(3, 8, dtype=torch.float16)
+    oc.scatter_into_peer(wide, local, 1, 2, 8, 5)  # columns 1..2 land at columns 5..6 of an 8-wide peer
+    assert wide[:, 5:7].tolist() == local[:, 1:3].tolist() and wide.sum() == local[:, 1:3].sum()
+
+
+def test_full_full_allscatter_gives_every_rank_the_full_product():
+    world, M, K, N = 2, 64, 32, 128
+    g = torch.Generator().manual_seed(0)
+    A, B = torch.randn(M, K, generator=g).half(), (torch.randn(K, N, generator=g) / K**0.5).half()
+    Cs = [torch.zeros(M, N, dtype=torch.float16) for _ in range(world)]
+    specs = []
+    for r in range(world):
+        s = resolve_pattern_execution(A, B, Cs[r], rank=r, world_size=world, b_layout="full", c_layout="full")
+        specs.append(dict(src_col_offset=s.scatter_src_col_offset, cols=s.scatter_cols,
+                          dst_ld=s.scatter_dst_leading_dim, dst_col_offset=s.scatter_dst_col_offset))
+    oc.gemm_allscatter([A] * world, [B] * world, Cs, specs)
+    want = (A.float() @ B.float()).half()
+    assert torch.equal(Cs[0], want) and torch.equal(Cs[1], want)
+
+
+def test_allgather_layout_and_directions():
+    M, N = 4, 3
+    outs = [torch.zeros(3 * M, N) for _ in range(3)]
+    for r in range(3):
+        outs[r][r * M:(r + 1) * M] = r + 1  # each rank's own block is resident
+    oc.allgather_exchange(outs, rank=1, M=M, push=True, pull=False)
+    assert all(torch.all(outs[p][M:2 * M] == 2) for p in range(3))  # rank 1's block is everywhere
+    assert torch.all(outs[1][:M] == 0) and torch.all(outs[1][2 * M:] == 0)  # nothing came in
+    oc.allgather_exchange(outs, rank=1, M=M, push=False, pull=True)
+    assert outs[1][:, 0].tolist() == [1.0] * M + [2.0] * M + [3.0] * M  # [block_rank0 | block_rank1 | block_rank2]
+
+
+def test_reduce_is_exact_fp32_then_one_rounding_owner_first():
+    big, small = 2.0**24, 1.0
+    # fp32: (big + small) + small == big, but (small + small) + big == big + 2: order is observable
+    partials = [torch.tensor([[big], [small]]), torch.tensor([[small], [big]]), torch.tensor([[small], [small]])]
+    partials = [p.repeat(1, 1) for p in partials]  # rows: shard 0 = row 0 (owner 0); world 3 needs 3 rows
+    partials = [torch.cat([p, torch.zeros(1, 1)]) for p in partials]
+    out0 = oc.reduce_rows(partials, 0, torch.float32)  # big first: big + 1 + 1 -> big (each +1 is lost)
+    assert out0.item() == big
+    out1 = oc.reduce_rows(partials, 1, torch.float32)  # owner 1 first: big, then rank 0: +1 lost, rank 2: +1 lost
+    assert out1.item() == big
+    swapped = [partials[2], partials[1], partials[0]]
+    assert oc.reduce_rows(swapped, 0, torch.float32).item() == big + 2  # small + small first, then big: exact
+    # rounding happens once, after the fp32 sum
+    a = torch.tensor([[1.0 + 2.0**-11]], dtype=torch.float32)
+    b = torch.tensor([[2.0**-11]], dtype=torch.float32)
+    assert oc.reduce_rows([a, b][:1] + [b][:0], 0, torch.float16).item() == 1.0  # single addend: tie rounds to even
+    two = oc.reduce_rows([torch.cat([a, a]), torch.cat([b, b])], 0, torch.float16)
+    assert two.item() == float(torch.tensor(1.0 + 2.0**-10).half())  # the sum is representable: no double rounding
+    assert oc.expected_counters([256, 128], epoch=3) == [768, 384]
