@@ -88,7 +88,8 @@ typedef struct tccl_gemm_desc {
   float alpha;       /* applied to the fp32 accumulator (fp8: scale_a * scale_b) */
   int32_t block_m, block_n, group_m; /* plan tile and swizzle band: 128/128/8 or 256/128/8 */
   int32_t num_wgs;   /* GEMM workgroups; 0 = library default for the device */
-  int32_t reserved[3];
+  int32_t macro_tile; /* output tile one workgroup computes: 0 = choose by shape, 128, or 256 */
+  int32_t reserved[2];
 } tccl_gemm_desc;
 
 /* ---- per-launch synchronisation words ------------------------------------------------

@@ -63,6 +63,7 @@ def gemm_desc(
     group_m: int = 8,
     alpha: float = 1.0,
     num_wgs: int = 0,
+    macro_tile: int = 0,
 ) -> _lib.GemmDesc:
     if not (A.is_cuda and B.is_cuda and C_out.is_cuda):
         raise ValueError("GEMM operands must be device tensors")
@@ -82,6 +83,7 @@ def gemm_desc(
     d.alpha = float(alpha)
     d.block_m, d.block_n, d.group_m = int(block_m), int(block_n), int(group_m)
     d.num_wgs = int(num_wgs)
+    d.macro_tile = int(macro_tile)
     return d
 
 

@@ -54,7 +54,8 @@ class GemmDesc(C.Structure):
         ("block_n", C.c_int32),
         ("group_m", C.c_int32),
         ("num_wgs", C.c_int32),
-        ("reserved", C.c_int32 * 3),
+        ("macro_tile", C.c_int32),
+        ("reserved", C.c_int32 * 2),
     ]
 
 

@@ -15,7 +15,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 OUT = HERE.parent / "libtileccl_hip.so"
 SOURCES = [HERE / "tccl_api.hip"]
-HEADERS = [HERE / "tccl_device.h", HERE / "tccl_gemm.h", HERE / "tccl_comm.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
+HEADERS = [HERE / "tccl_device.h", HERE / "tccl_gemm.h", HERE / "tccl_gemm256.h", HERE / "tccl_comm.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
 
 FLAGS = [
     "--offload-arch=gfx950",

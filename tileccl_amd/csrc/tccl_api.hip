@@ -9,6 +9,7 @@
 #include "../../include/tileccl_hip.h"
 #include "tccl_comm.h"
 #include "tccl_gemm.h"
+#include "tccl_gemm256.h"
 
 namespace {
 
@@ -92,6 +93,53 @@ __global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::S
   }
 }
 
+// Large-tile GEMM: 512 threads, one workgroup per CU, both LDS stages resident.
+template <typename InT, typename OutT>
+__global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl::Macro m) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
+  __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
+  tccl::SignalArgs s;
+  s.mode = tccl::kSignalNone;
+  tccl::PullArgs no_pull;
+  no_pull.peers = 0;
+  tccl::Gemm256<InT, OutT>(g, no_pull, -1, stage0, stage1, nullptr, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
+#endif
+}
+
+// Large-tile GEMM whose workgroups, once their tiles are stored (and pushed to the peers
+// from the epilogue), turn into the communication role.  The tile fills a CU's LDS and
+// registers, so no separate communication workgroup could share the CU with it; instead
+// every workgroup produces first and moves data afterwards.  No workgroup waits before its
+// own tiles are published and the grid never exceeds the CU count, so every wait is on a
+// workgroup that is running.  `push` and `comm` are read from the argument block at their
+// point of use (late_kernarg), never through the parameter itself.
+struct Fused256Args {
+  tccl::GemmArgs g;
+  tccl::SignalArgs s;
+  tccl::Macro m;
+  int64_t* trace_start;
+  tccl::PullArgs pull;
+  tccl::PushArgs push;
+  tccl::CommArgs comm;
+};
+
+template <typename InT, typename OutT>
+__global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
+  __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
+  __shared__ __attribute__((aligned(16))) char pull0[tccl::kPullSlotBytes];
+  __shared__ __attribute__((aligned(16))) char pull1[tccl::kPullSlotBytes];
+  if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
+  tccl::Gemm256<InT, OutT>(f.g, f.pull, (int)offsetof(Fused256Args, push), stage0, stage1, pull0, pull1)
+      .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
+  __syncthreads();
+  const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));
+  tccl::comm_role<tccl::kThreads256>(c, (int)blockIdx.x, (int)gridDim.x, (int*)stage1);
+#endif
+}
+
 __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   __shared__ int word[4];
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
@@ -122,6 +170,8 @@ int check_gemm(const tccl_gemm_desc* d) {
   if (d->block_m <= 0 || d->block_n <= 0 || d->group_m <= 0) return fail(TCCL_ERR_INVALID, "gemm: block_m, block_n, group_m must be positive");
   if (d->block_m % tccl::kTile || d->block_n % tccl::kTile)
     return fail(TCCL_ERR_UNSUPPORTED, "gemm: plan tile %dx%d must be a multiple of 128x128", d->block_m, d->block_n);
+  if (d->macro_tile != 0 && d->macro_tile != 128 && d->macro_tile != 256)
+    return fail(TCCL_ERR_INVALID, "gemm: macro_tile=%d must be 0, 128 or 256", d->macro_tile);
   const size_t isz = dtype_size(d->in_dtype), osz = dtype_size(d->out_dtype);
   if (!isz || !osz) return fail(TCCL_ERR_INVALID, "gemm: unknown dtype");
   if (d->in_dtype == TCCL_F32) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp32 inputs have no MFMA kernel here");
@@ -260,6 +310,127 @@ int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tcc
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 
+// ---- large-tile path ----------------------------------------------------------------------------
+bool plan_tile_fits_macro(const tccl_gemm_desc* d) {
+  return (d->block_m == 128 || d->block_m == 256) && (d->block_n == 128 || d->block_n == 256);
+}
+
+// 256 x 256 tiles pay off once there are enough of them to occupy most CUs; below that
+// the 128 x 128 kernel spreads the work over more workgroups.
+bool use_macro(const tccl_gemm_desc* d, const tccl_device_info& dev) {
+  if (!plan_tile_fits_macro(d)) return false;
+  if (d->macro_tile == 128) return false;
+  if (d->macro_tile == 256) return true;
+  const int64_t tiles = (int64_t)((d->M + 255) / 256) * ((d->N + 255) / 256);
+  return tiles * 2 >= dev.compute_units;
+}
+
+tccl::Macro build_macro(const tccl_gemm_desc* d, const tccl_device_info& dev, int num_wgs) {
+  tccl::Macro m;
+  m.rows = (d->M + 255) / 256;
+  m.cols = (d->N + 255) / 256;
+  const int band_rows = d->group_m * d->block_m / 256;
+  m.rows_per_band = band_rows > 0 ? band_rows : 1;
+  m.xcds = dev.xcds;
+  // Ids an XCD takes from each block: its share of the tiles in flight, in whole band columns.
+  const int total = m.rows * m.cols;
+  const int in_flight = total < num_wgs ? total : num_wgs;
+  int span = in_flight / (dev.xcds > 0 ? dev.xcds : 1);
+  span = span / m.rows_per_band * m.rows_per_band;
+  m.span = span > 0 ? span : 1;
+  return m;
+}
+
+int default_macro_wgs(const tccl_gemm_desc* d, const tccl_device_info& dev) {
+  const int total = ((d->M + 255) / 256) * ((d->N + 255) / 256);
+  int n = d->num_wgs > 0 ? d->num_wgs : dev.compute_units;
+  if (n > total) n = total;
+  return n < 1 ? 1 : n;
+}
+
+template <typename InT, typename OutT>
+int launch_gemm256_t(const tccl::GemmArgs& g, const tccl::Macro& m, int wgs, hipStream_t stream) {
+  hipLaunchKernelGGL((gemm256_kernel<InT, OutT>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, g, m);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int launch_gemm256(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tccl::Macro& m, int wgs, hipStream_t stream) {
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_gemm256_t<_Float16, _Float16>(g, m, wgs, stream);
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_gemm256_t<_Float16, float>(g, m, wgs, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_gemm256_t<__bf16, __bf16>(g, m, wgs, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_gemm256_t<__bf16, float>(g, m, wgs, stream);
+  return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
+}
+
+template <typename InT, typename OutT>
+int launch_fused256_t(const Fused256Args& f, int wgs, hipStream_t stream) {
+  hipLaunchKernelGGL((fused256_kernel<InT, OutT>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs, hipStream_t stream) {
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_fused256_t<_Float16, _Float16>(f, wgs, stream);
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused256_t<_Float16, float>(f, wgs, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused256_t<__bf16, __bf16>(f, wgs, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused256_t<__bf16, float>(f, wgs, stream);
+  return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
+}
+
+// The pull half of a TileGroup all-gather, as the large-tile K loop performs it in the
+// background.  Returns false when there is nothing of the kind to do.
+bool build_pull(const tccl::CommArgs& c, tccl::PullArgs* p) {
+  memset(p, 0, sizeof *p);
+  if (c.op != tccl::kOpAllGather || c.granularity != tccl::kPerGroup || !(c.directions & tccl::kDirPull) || c.world <= 1) return false;
+  if (!c.row_ends || !c.tile_counts || !c.counter) return false;
+  const int64_t row_bytes = (int64_t)c.N * c.esize;
+  const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
+  if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
+  p->peers = c.world - 1;
+  p->rank = c.rank;
+  p->heap_bases = c.heap_bases;
+  p->block0_off = (int64_t)(uintptr_t)c.out - c.heap_bases[c.rank];
+  p->block_bytes = block_bytes;
+  p->pitch = (uint32_t)c.ld_out_bytes;
+  p->upr = (uint32_t)(row_bytes / 16);
+  p->units = (uint32_t)c.M * p->upr;
+  p->pieces = (int)((p->units + 63) / 64);
+  p->counter = c.counter;
+  p->row_ends = c.row_ends;
+  p->tile_counts = c.tile_counts;
+  p->n_groups = c.n_groups;
+  p->epoch = c.epoch;
+  p->barrier = c.barrier;
+  p->trace_done_clock = c.trace_done_clock;
+  p->fault = c.fault;
+  p->spin_ticks = c.spin_ticks;
+  return true;
+}
+
+// The push half of an all-scatter / all-gather, as the large-tile epilogue performs it.
+// Returns false when the operation has no push to fold (reduce-scatter, push not asked for).
+bool build_push(const tccl::CommArgs& c, const tccl::GemmArgs& g, tccl::PushArgs* p) {
+  memset(p, 0, sizeof *p);
+  if (!(c.directions & tccl::kDirPush) || c.world <= 1) return false;
+  if (c.op != tccl::kOpAllScatter && c.op != tccl::kOpAllGather) return false;
+  const int64_t mine = c.heap_bases[c.rank];
+  for (int q = 0; q < c.world; ++q)
+    if (q != c.rank) p->base[p->n++] = (char*)g.C + (c.heap_bases[q] - mine);
+  if (c.op == tccl::kOpAllScatter) {
+    p->col_lo = c.src_col_off;
+    p->col_hi = c.src_col_off + c.cols;
+    p->col_shift = c.dst_col_off - c.src_col_off;
+    p->ld = c.dst_ld;
+  } else {
+    p->col_lo = 0;
+    p->col_hi = g.N;
+    p->col_shift = 0;
+    p->ld = g.ldc;
+  }
+  return true;
+}
+
 int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
   if (wgs < 1) wgs = 1;
   hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
@@ -277,6 +448,39 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
   tccl::SignalArgs s;
   memset(&s, 0, sizeof s);
   int64_t* trace_start = sync ? sync->trace_start_clock : nullptr;
+  if (use_macro(d, dev)) {
+    const int wgs = default_macro_wgs(d, dev);
+    const tccl::Macro m = build_macro(d, dev, wgs);
+    if (variant == TCCL_S0_BULK) {
+      int rc = launch_gemm256(d->in_dtype, d->out_dtype, g, m, wgs, stream);
+      if (rc) return rc;
+      c.granularity = tccl::kBulk;
+      if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
+      return launch_comm(c, bulk_comm_wgs(dev), stream);
+    }
+    Fused256Args f;
+    f.g = g;
+    f.m = m;
+    f.trace_start = trace_start;
+    if (variant == TCCL_S1_TILE) {
+      s.mode = tccl::kSignalTile;
+      s.locks = sync->locks;
+      c.granularity = tccl::kPerTile;
+    } else {
+      s.mode = tccl::kSignalGroup;
+      s.counter = sync->counter;
+      s.group_table = sync->group_table;
+      c.granularity = tccl::kPerGroup;
+    }
+    f.s = s;
+    // Pushes leave from the epilogue; what remains for the communication role are the
+    // pulls (and, for a reduce-scatter, the reductions).
+    if (build_push(c, g, &f.push)) c.directions &= ~tccl::kDirPush;
+    if (build_pull(c, &f.pull)) c.directions &= ~tccl::kDirPull;
+    if (c.op != tccl::kOpReduceScatter && !(c.directions & (tccl::kDirPush | tccl::kDirPull))) c.op = tccl::kOpNone;
+    f.comm = c;
+    return launch_fused256(d->in_dtype, d->out_dtype, f, wgs, stream);
+  }
   if (variant == TCCL_S0_BULK) {
     tccl::CommArgs none;
     memset(&none, 0, sizeof none);
@@ -399,6 +603,10 @@ int tccl_gemm(const tccl_gemm_desc* d, void* stream) {
   build_gemm_args(d, dev, &g);
   tccl::SignalArgs s;
   memset(&s, 0, sizeof s);
+  if (use_macro(d, dev)) {
+    const int wgs = default_macro_wgs(d, dev);
+    return launch_gemm256(d->in_dtype, d->out_dtype, g, build_macro(d, dev, wgs), wgs, (hipStream_t)stream);
+  }
   tccl::CommArgs none;
   memset(&none, 0, sizeof none);
   return launch_fused(d->in_dtype, d->out_dtype, g, s, none, default_gemm_wgs(d, dev, g.tile_rows * g.tile_cols), 0, nullptr,

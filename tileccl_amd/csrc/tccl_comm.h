@@ -86,26 +86,26 @@ TCCL_D u32x4 ld16(__amdgpu_buffer_rsrc_t w, uint32_t off) { return __builtin_amd
 template <int kPolicy>
 TCCL_D void st16(__amdgpu_buffer_rsrc_t w, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, w, off, 0, kPolicy); }
 
-constexpr int kThreadsComm = 256;  // threads of a communication workgroup
+constexpr int kThreadsComm = 256;  // threads of a stand-alone communication workgroup
 constexpr int kCommUnroll = 8;     // 16-byte accesses a thread keeps in flight
 
 // ---- copy: units [u_lo, u_hi) of the rectangle, one source slice, any number of targets ----
 // kPolicy is the cache policy of both sides: kCoherent inside fused launches (the source
 // was just written by other workgroups, the target will be read by a peer), kStreaming
 // for the stand-alone bulk kernel.
-template <int kPolicy>
+template <int kPolicy, int kThreads>
 TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const int tid = threadIdx.x;
   const int src_rank = __builtin_ctz(x.src_ranks);
   const __amdgpu_buffer_rsrc_t src = window(a.heap_bases[src_rank] + x.src_off);
   const bool flat = (x.src_pitch == (int64_t)x.upr * 16) && (x.dst_pitch == x.src_pitch);
   const uint32_t sp = (uint32_t)x.src_pitch, dp = (uint32_t)x.dst_pitch;
-  for (int u0 = u_lo; u0 < u_hi; u0 += kThreadsComm * kCommUnroll) {
+  for (int u0 = u_lo; u0 < u_hi; u0 += kThreads * kCommUnroll) {
     u32x4 v[kCommUnroll];
     uint32_t doff[kCommUnroll];
 #pragma unroll
     for (int k = 0; k < kCommUnroll; ++k) {
-      const int u = u0 + tid + k * kThreadsComm;
+      const int u = u0 + tid + k * kThreads;
       uint32_t soff;
       if (flat) {
         soff = (uint32_t)u * 16u;
@@ -123,7 +123,7 @@ TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
       const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[q] + x.dst_off);
 #pragma unroll
       for (int k = 0; k < kCommUnroll; ++k)
-        if (u0 + tid + k * kThreadsComm < u_hi) st16<kPolicy>(dst, doff[k], v[k]);
+        if (u0 + tid + k * kThreads < u_hi) st16<kPolicy>(dst, doff[k], v[k]);
     }
   }
 }
@@ -181,7 +181,7 @@ constexpr int kReduceUnroll = 2;
 
 // Sum order: the owner's addend first, then the other ranks in ascending order
 // (tile_reduce_scatter: local chunk, then peers ascending; collectives.py:766-781).
-template <typename PT, typename OT, int kPolicy>
+template <typename PT, typename OT, int kPolicy, int kThreads>
 TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   constexpr uint32_t kSrcUnit = 8 * sizeof(PT);
   const int tid = threadIdx.x;
@@ -189,12 +189,12 @@ TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[dst_rank] + x.dst_off);
   const __amdgpu_buffer_rsrc_t first = window(a.heap_bases[x.first_rank] + x.src_off);
   const uint32_t sp = (uint32_t)x.src_pitch, dp = (uint32_t)x.dst_pitch;
-  for (int u0 = u_lo; u0 < u_hi; u0 += kThreadsComm * kReduceUnroll) {
+  for (int u0 = u_lo; u0 < u_hi; u0 += kThreads * kReduceUnroll) {
     float acc[kReduceUnroll][8];
     uint32_t soff[kReduceUnroll], doff[kReduceUnroll];
 #pragma unroll
     for (int k = 0; k < kReduceUnroll; ++k) {
-      const int u = u0 + tid + k * kThreadsComm;
+      const int u = u0 + tid + k * kThreads;
       const uint32_t r = (uint32_t)u / (uint32_t)x.upr, c = (uint32_t)u - r * (uint32_t)x.upr;
       soff[k] = r * sp + c * kSrcUnit;
       doff[k] = r * dp + c * 16u;
@@ -214,36 +214,37 @@ TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
     }
 #pragma unroll
     for (int k = 0; k < kReduceUnroll; ++k)
-      if (u0 + tid + k * kThreadsComm < u_hi) st16<kPolicy>(dst, doff[k], pack8<OT>(acc[k]));
+      if (u0 + tid + k * kThreads < u_hi) st16<kPolicy>(dst, doff[k], pack8<OT>(acc[k]));
   }
 }
 
-template <int kPolicy>
+template <int kPolicy, int kThreads>
 TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const int key = a.partial_dtype * 4 + a.out_dtype;
   switch (key) {
-    case kF32 * 4 + kF16: run_reduce_t<float, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
-    case kF32 * 4 + kBF16: run_reduce_t<float, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
-    case kF16 * 4 + kF16: run_reduce_t<_Float16, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
-    case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
-    case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16, kPolicy>(a, x, u_lo, u_hi); break;
-    case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16, kPolicy>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kF16: run_reduce_t<float, _Float16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kBF16: run_reduce_t<float, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kF16: run_reduce_t<_Float16, _Float16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
     default: break;
   }
 }
 
+template <int kThreads>
 TCCL_D void run_xfer(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   const bool fused = a.granularity != kBulk;
   if (x.reduce) {
     if (fused)
-      run_reduce<kCoherent>(a, x, u_lo, u_hi);
+      run_reduce<kCoherent, kThreads>(a, x, u_lo, u_hi);
     else
-      run_reduce<kStreaming>(a, x, u_lo, u_hi);
+      run_reduce<kStreaming, kThreads>(a, x, u_lo, u_hi);
   } else {
     if (fused)
-      run_copy<kCoherent>(a, x, u_lo, u_hi);
+      run_copy<kCoherent, kThreads>(a, x, u_lo, u_hi);
     else
-      run_copy<kStreaming>(a, x, u_lo, u_hi);
+      run_copy<kStreaming, kThreads>(a, x, u_lo, u_hi);
   }
 }
 
@@ -388,6 +389,7 @@ TCCL_D bool rs_not_mine(const CommArgs& a, int row) {
 // sources are ready or soon will be, independent of this rank's GEMM), then pushes /
 // reductions in production order.  Workgroup w takes tasks w, w + n, w + 2n, ...; no
 // GEMM workgroup ever waits on a communication workgroup, so the order is deadlock-free.
+template <int kThreads = kThreadsComm>
 TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
   if (a.op == kOpNone || num_wgs <= 0) return;
   Waiter wait{a, lds_word, now_ticks() + a.spin_ticks};
@@ -423,7 +425,7 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
       }
       Xfer x;
       const int r0 = tc.m * a.block_m, c0 = tc.n * a.block_n;
-      if (ok && make_xfer(a, pull, peer, r0, r0 + a.block_m, c0, c0 + a.block_n, x)) run_xfer(a, x, 0, x.rows * x.upr);
+      if (ok && make_xfer(a, pull, peer, r0, r0 + a.block_m, c0, c0 + a.block_n, x)) run_xfer<kThreads>(a, x, 0, x.rows * x.upr);
     }
     return;
   }
@@ -462,7 +464,7 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
       const int units = x.rows * x.upr;
       const int lo = local * units_per_task;
       const int hi = lo + units_per_task < units ? lo + units_per_task : units;
-      if (lo < hi) run_xfer(a, x, lo, hi);
+      if (lo < hi) run_xfer<kThreads>(a, x, lo, hi);
     }
     if (a.granularity == kPerGroup) task_done(a, g, tasks_g * tasks_factor);
   }

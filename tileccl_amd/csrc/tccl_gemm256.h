@@ -1,0 +1,610 @@
+// Large-tile MFMA GEMM for gfx950: one workgroup of 512 threads (8 wavefronts, 2 x 4)
+// produces a 256 x 256 macro tile, K consumed 64 at a time.
+//
+// Why a second GEMM: measured on MI355X, a CU's LDS takes ~78 B/clk of writes and 256 B/clk
+// of reads.  A 128 x 128 tile needs 32 KB of operands written per 512 MFMA cycles (64 B/clk,
+// most of what the LDS accepts); at 256 x 256 the same bytes feed four times the math.  A
+// wave owns 128 x 64 outputs (128 fp32 accumulators per lane), which also cuts the LDS
+// reads per MFMA.
+//
+// Global -> LDS: `buffer_load_dwordx4 ... lds` copies 16 bytes per lane straight into LDS (no
+// staging registers, no ds_write).  The hardware places lane l's bytes at base + 16*l, so the
+// LDS layout is fixed to "lanes in order" and the swizzle that keeps the MFMA reads free of
+// bank conflicts is applied on the global side, by choosing which 16-byte chunk a lane
+// fetches:
+//   A stage: row-major, 128 B per row (64 k); chunk kc of row r lives in slot kc ^ ((r >> 1) & 7).
+//   B stage: natural [k][n], 512 B per k row; chunk c of row k lives in slot c ^ (4 * (k & 3)).
+// A operands are read with ds_read_b128 (8 consecutive k of one row).  B operands are read
+// with ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of 4 consecutive n of
+// k row i/4 at column block i%4, and lane j receives 4 consecutive k for column j; two reads
+// give a lane the 8 consecutive k of v_mfma_f32_32x32x16.
+//
+// Pipeline: LDS holds two stages.  The loads of step kt+1 are issued, woven between the
+// MFMAs of step kt, into the stage step kt-1 has just left; `s_waitcnt vmcnt(0)` and one
+// barrier close the step, so a load has a full step of math (~2000 cycles) to land.
+//
+// The swapped-operand MFMA and the slab-wise epilogue are those of tccl_gemm.h.
+//
+// A macro tile covers (256/block_m) x (256/block_n) plan tiles; when it is stored, each of
+// them is published under its swizzled tile id, so locks / group_table keep the
+// reference's numbering (tileccl/kernels/gemm.py:118-123, tileccl_v2/tile_group.py:229-234).
+#pragma once
+
+#include "tccl_comm.h"
+#include "tccl_gemm.h"
+
+namespace tccl {
+
+constexpr int kMacro = 256;
+constexpr int kThreads256 = 512;
+constexpr int kARow256 = 128;                              // A: bytes per row of one stage (64 k)
+constexpr int kAStage256 = kMacro * kARow256;              // 32 768 B
+constexpr int kBPitch256 = 512;                            // B: bytes per k row (256 columns)
+constexpr int kBStage256 = kBK * kBPitch256;               // 32 768 B
+constexpr int kStage256 = kAStage256 + kBStage256;         // A then B
+constexpr int kLds256 = 2 * kStage256;                     // two stages: 131 072 B (two arrays)
+
+struct Macro {
+  int rows, cols;        // macro tile grid
+  int rows_per_band;     // macro rows that form one swizzle band of the plan
+  int xcds, span;        // slot -> macro id remap
+};
+
+// Where the epilogue sends a finished tile besides C: the same rows of every listed target,
+// columns [col_lo, col_hi) of C landing at column + col_shift.  This is the push half of an
+// all-scatter / all-gather folded into the GEMM: the tile goes out from the staging LDS it
+// already sits in, instead of being written, signalled, re-read and copied by a second party
+// (reference: the per-tile scatter of patterns/_helpers.py:86-199, tile_allgather of
+// primitives/collectives.py:613-663).
+constexpr int kMaxPush = 7;
+struct PushArgs {
+  int n;               // number of targets; 0: the epilogue writes C only
+  int col_lo, col_hi;  // columns of C that travel
+  int col_shift;       // target column = C column + col_shift
+  int64_t ld;          // target pitch in elements
+  char* base[kMaxPush];  // address of C's (row 0, column 0) inside each target
+};
+
+// The pull half of an all-gather, carried out in the shadow of the K loop (TileGroup variant).
+// A peer's block is cut into 1 KiB pieces (64 lanes x 16 bytes); wavefront w of the launch
+// owns pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid
+// sweeps a contiguous stretch of the block.  Each K step a wavefront stores the piece it
+// fetched during the previous step and fetches the next one straight into LDS; a piece is
+// fetched only once the TileGroups covering its rows are complete on the peer
+// (counter[g] >= epoch * tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66),
+// which is found out by a counter fetch that is itself left in flight for one K step.  What the
+// K loops did not get to is finished after the last tile, with bounded waits.
+// Groups must cover the block's rows in ascending order (build_tile_group_plan emits them so:
+// tileccl_v2/tile_group.py:244-301).
+struct PullArgs {
+  int peers;                   // peers pulled from; 0 turns the background pull off
+  int rank;
+  const int64_t* heap_bases;
+  int64_t block0_off;          // slice offset of rank 0's block
+  int64_t block_bytes;         // distance between consecutive ranks' blocks (rows * pitch)
+  uint32_t pitch;              // bytes per row
+  uint32_t upr;                // 16-byte units per row
+  uint32_t units;              // units per block (rows * upr)
+  int pieces;                  // pieces per block: ceil(units / 64)
+  const int32_t* counter;      // this rank's TileGroup counters; a peer's sit at the same slice offset
+  const int32_t* row_ends;
+  const int32_t* tile_counts;
+  int n_groups, epoch;
+  int32_t* barrier;            // every barrier[g] grows by the grid size once all shares are stored
+  int64_t* trace_done_clock;
+  int64_t* fault;
+  int64_t spin_ticks;
+};
+constexpr int kPullPieceBytes = 8 * 1024;                   // one 1 KiB landing slot per wavefront
+constexpr int kPullSlotBytes = kPullPieceBytes + 8 * 256;   // plus 256 B per wavefront for a fetched counter
+
+TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
+  const int per_band = m.rows_per_band * m.cols;
+  const int band = id / per_band;
+  const int first = band * m.rows_per_band;
+  const int height = (m.rows - first) < m.rows_per_band ? (m.rows - first) : m.rows_per_band;
+  const int within = id - band * per_band;
+  TileCoord c;
+  c.m = first + within % height;
+  c.n = within / height;
+  return c;
+}
+
+// Device pass only: the host pass needs the launch signature, not the body.
+#if defined(__HIP_DEVICE_COMPILE__)
+// A by-value kernel argument read where it is used instead of at kernel entry: arguments
+// that only the epilogue or the communication role need would otherwise sit in scalar
+// registers (and spill into vector registers) all through the K loop.  The empty asm hides
+// the address from the optimiser until control reaches this point.
+template <typename T>
+TCCL_D T late_kernarg(int offset) {
+  typedef const __attribute__((address_space(4))) char* KernargPtr;
+  KernargPtr p = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr() + offset;
+  asm volatile("" : "+s"(p));
+  T v;
+  __builtin_memcpy(&v, p, sizeof(T));
+  return v;
+}
+
+template <typename InT, typename OutT>
+struct Gemm256 {
+  typedef typename Mfma<InT>::Vec Vec;
+
+  const GemmArgs& g;
+  const PullArgs& pa;
+  const int push_offset;  // byte offset of a PushArgs in the kernel arguments; < 0: no push
+  // The two pipeline stages are two separate __shared__ arrays: loads that write LDS directly
+  // are tracked per LDS variable, so a read of one stage need not wait for a load into the other.
+  char* lds;   // stage 0 (also the epilogue's staging area)
+  char* lds1;  // stage 1
+  char* bg0;   // landing slots of the background pull, one array per K-step parity
+  char* bg1;
+  const int tid, lane, wave, wm, wn;
+
+  TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, char* stage0, char* stage1,
+                 char* pull0, char* pull1)
+      : g(args), pa(pull_args), push_offset(push_args_offset), lds(stage0), lds1(stage1), bg0(pull0), bg1(pull1), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+        wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
+
+  typedef __attribute__((address_space(3))) void LdsVoid;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 LdsQuad;
+
+  // Where this lane's four A pieces and four B pieces of a K step come from (byte offsets
+  // into the buffer resources at K step 0).  Piece i of wave w fills
+  //   A rows 8*(4w+i) .. +7      (lane l: row + l/8, slot l%8)
+  //   B k rows 2*(4w+i), +1      (lane l: k row + l/32, slot l%32)
+  struct Source {
+    __amdgpu_buffer_rsrc_t a, b;
+    uint32_t off_a[4], off_b[4];
+    uint32_t step_a, step_b;
+  };
+
+  static TCCL_D uint32_t clamp_u32(int64_t v) { return v > 0xffffffffll ? 0xffffffffu : (v < 0 ? 0u : (uint32_t)v); }
+
+  TCCL_D Source make_source(int row0, int col0) const {
+    constexpr int kEsz = sizeof(InT);
+    Source s;
+    const InT* A = (const InT*)g.A + (int64_t)row0 * g.lda;
+    const InT* B = (const InT*)g.B + col0;
+    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(g.M - 1 - row0) * g.lda + g.K) * kEsz), 0x00020000);
+    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (g.N - col0)) * kEsz), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * (4 * wave + i) + (lane >> 3);
+      const int kc = (lane & 7) ^ ((row >> 1) & 7);
+      s.off_a[i] = (uint32_t)(row * g.lda * kEsz + kc * 16);
+      const int k = 2 * (4 * wave + i) + (lane >> 5);
+      const int c = (lane & 31) ^ (4 * (k & 3));
+      s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
+    }
+    s.step_a = kBK * kEsz;
+    s.step_b = (uint32_t)(kBK * g.ldb * kEsz);
+    return s;
+  }
+
+  // Piece i of K step kt, straight into `stage`.  A chunks at k >= K are redirected past the
+  // end of the buffer so that they read as zero (B rows >= K already lie past it).
+  TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
+    const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);  // as in make_source
+    const bool dead = kt * kBK + kc * 8 >= g.K;
+    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + kt * s.step_a;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + 8 * (4 * wave + i) * kARow256), 16, oa, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + 2 * (4 * wave + i) * kBPitch256), 16,
+                                             s.off_b[i] + kt * s.step_b, 0, 0, 0);
+  }
+
+  // Per-lane LDS read addresses that do not depend on the k-chunk.
+  struct Reader {
+    uint32_t a_base;   // row of this lane in the A stage
+    uint32_t a_swz;    // XOR term of the A slot
+    uint32_t b_base0;  // B address for column block bj = 0 (bj = 1 is b_base0 ^ 64), k row of kk = 0, q = 0
+  };
+
+  TCCL_D Reader make_reader() const {
+    const int half = lane >> 5, l32 = lane & 31, i16 = lane & 15, grp = (lane >> 4) & 1;
+    const int t = i16 >> 2, cq = i16 & 3;
+    Reader r;
+    r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
+    r.a_swz = (uint32_t)((l32 >> 1) & 7);
+    const int chunk = (wn * 8 + grp * 2 + (cq >> 1)) ^ (4 * t);
+    r.b_base0 = (uint32_t)(kAStage256 + (8 * half + t) * kBPitch256 + chunk * 16 + (cq & 1) * 8);
+    return r;
+  }
+
+  TCCL_D void load_frags(const char* stage, const Reader& r, int kk, Vec (&fa)[4], Vec (&fb)[2]) const {
+    const int half = lane >> 5;
+    const char* pa = stage + r.a_base + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) fa[b] = *(const Vec*)(pa + b * 32 * kARow256);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch256;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)pb);
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch256));
+      const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      fb[b] = __builtin_bit_cast(Vec, both);
+    }
+  }
+
+  // ---- background pull ---------------------------------------------------------------------------
+  struct PullState {
+    int next_slot, next_lp;  // next piece of this wavefront: peer slot, piece inside the block
+    int stride;              // wavefronts in the grid
+    int slot;                // peer slot that the bases and the readiness cache describe (-1: none)
+    int gidx;                // first TileGroup of that peer not yet known complete
+    uint32_t ready_units;    // units [0, ready_units) of that peer's block may be fetched
+    int64_t src_base, dst_base;
+    int64_t counter_base;    // address of that peer's counter words
+    int probe_group;         // group whose counter was fetched (into the landing slot) during the previous step; -1: none
+    int pending_lp;          // piece fetched into LDS during the previous step (-1: none)
+    const char* pending_lds; // where it landed
+    int lds_off;             // this wavefront's landing slot inside a slot array
+  };
+
+  // Values that are the same in every lane but that the compiler cannot prove so (loaded
+  // through a pointer, derived from threadIdx) are moved to scalar registers explicitly;
+  // otherwise each buffer descriptor built from them costs a per-lane loop.
+  static TCCL_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+  // Read-only tables (plan rows, tile counts, slice bases) through the scalar path.
+  template <typename T>
+  static TCCL_D T table(const T* p, int i) {
+    return ((const __attribute__((address_space(4))) T*)p)[i];
+  }
+  static TCCL_D int64_t uniform64(int64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+  }
+
+  TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
+    PullState st;
+    const int w = uniform(wave);
+    st.lds_off = w * 1024;
+    st.stride = num_wgs * (kThreads256 / 64);
+    st.next_slot = 0;
+    st.next_lp = wg * (kThreads256 / 64) + w;
+    st.slot = -1;
+    st.gidx = 0;
+    st.ready_units = 0;
+    st.src_base = st.dst_base = st.counter_base = 0;
+    st.probe_group = -1;
+    st.pending_lp = -1;
+    st.pending_lds = nullptr;
+    pull_normalise(st, a);
+    return st;
+  }
+
+  // Fetch the first counter before the first tile's prologue, so that the first K step can
+  // already fetch a piece.  `landing` is the slot array that K step 0 reads.
+  TCCL_D void pull_prime(PullState& st, const PullArgs& a, char* landing) const {
+    if (a.peers == 0 || st.next_slot >= a.peers) return;
+    pull_select(st, a, st.next_slot);
+    pull_probe(st, a, landing);
+  }
+
+  TCCL_D void pull_probe(PullState& st, const PullArgs& a, char* landing) const {
+    if (st.gidx >= a.n_groups) return;
+    // every lane fetches the same word
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter_base), (LdsVoid*)(landing + kPullPieceBytes + (st.lds_off >> 2)), 4,
+                                             (uint32_t)st.gidx * 4u, 0, 0, kCoherent);
+    st.probe_group = st.gidx;
+  }
+
+  TCCL_D void pull_normalise(PullState& st, const PullArgs& a) const {
+    while (st.next_lp >= a.pieces && st.next_slot < a.peers) {
+      st.next_lp -= a.pieces;
+      ++st.next_slot;
+    }
+  }
+
+  TCCL_D uint32_t pull_offset(const PullArgs& a, int lp, bool& valid) const {
+    const uint32_t u = (uint32_t)lp * 64u + (uint32_t)lane;
+    valid = u < a.units;
+    const uint32_t uu = valid ? u : 0u;  // idle lanes touch the block's first unit and store nothing
+    if (a.pitch == a.upr * 16u) return uu * 16u;
+    const uint32_t row = uu / a.upr;
+    return row * a.pitch + (uu - row * a.upr) * 16u;
+  }
+
+  TCCL_D uint32_t pull_last_unit(const PullArgs& a, int lp) const {
+    const uint32_t last = (uint32_t)lp * 64u + 63u;
+    return last < a.units ? last : a.units - 1u;
+  }
+
+  TCCL_D void pull_select(PullState& st, const PullArgs& a, int slot) const {
+    if (slot == st.slot) return;
+    const int peer = slot < a.rank ? slot : slot + 1;
+    st.slot = slot;
+    st.gidx = 0;
+    st.ready_units = 0;
+    st.probe_group = -1;
+    const int64_t rel = a.block0_off + (int64_t)peer * a.block_bytes;
+    const int64_t mine = table(a.heap_bases, a.rank), theirs = table(a.heap_bases, peer);
+    st.src_base = theirs + rel;
+    st.dst_base = mine + rel;
+    st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
+  }
+
+  TCCL_D void pull_store_pending(PullState& st, const PullArgs& a, const char* slot_lds) const {
+    bool valid;
+    const uint32_t off = pull_offset(a, st.pending_lp, valid);
+    const u32x4 v = *(const u32x4*)(slot_lds + lane * 16);
+    if (valid) st16<kStreaming>(window(st.dst_base), off, v);
+    st.pending_lp = -1;
+  }
+
+  TCCL_D void pull_group_done(PullState& st, const PullArgs& a, int g) const {
+    st.ready_units = (uint32_t)table(a.row_ends, g) * a.upr;
+    st.gidx = g + 1;
+  }
+
+  // The per-K-step slice of the pull; all control flow here is wavefront-uniform.
+  TCCL_D void pull_step(PullState& st, const PullArgs& a, char* load_lds, const char* store_lds) const {
+    if (a.peers == 0) return;
+    if (st.pending_lp >= 0) pull_store_pending(st, a, store_lds + st.lds_off);
+    if (st.probe_group >= 0) {
+      const int g = st.probe_group;
+      st.probe_group = -1;
+      const int32_t seen = uniform(*(const int32_t*)(store_lds + kPullPieceBytes + (st.lds_off >> 2)));
+      if (seen >= a.epoch * table(a.tile_counts, g)) pull_group_done(st, a, g);
+    }
+    if (st.next_slot >= a.peers) return;
+    if (st.next_slot != st.slot) {
+      pull_select(st, a, st.next_slot);
+      pull_probe(st, a, load_lds);
+      return;
+    }
+    if (pull_last_unit(a, st.next_lp) < st.ready_units) {
+      bool valid;
+      const uint32_t off = pull_offset(a, st.next_lp, valid);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(load_lds + st.lds_off), 16, off, 0, 0, kCoherent);
+      st.pending_lp = st.next_lp;
+      st.pending_lds = load_lds + st.lds_off;
+      st.next_lp += st.stride;
+      pull_normalise(st, a);
+    }
+    pull_probe(st, a, load_lds);  // look ahead: the next group's counter
+  }
+
+  // Wait (bounded) until units [0, last] of the selected peer's block may be fetched.
+  TCCL_D bool pull_wait_ready(PullState& st, const PullArgs& a, uint32_t last, int64_t deadline) const {
+    while (last >= st.ready_units) {
+      if (st.gidx >= a.n_groups) return false;
+      const int32_t need = a.epoch * table(a.tile_counts, st.gidx);
+      const __amdgpu_buffer_rsrc_t words = window(st.counter_base);
+      for (;;) {
+        const int32_t seen = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(words, (uint32_t)st.gidx * 4u, 0, kCoherent);
+        if (uniform(seen) >= need) break;
+        if (now_ticks() > deadline) return false;
+        __builtin_amdgcn_s_sleep(8);
+      }
+      pull_group_done(st, a, st.gidx);
+    }
+    return true;
+  }
+
+  // After the last tile: store what is in flight, move the remaining pieces, report.
+  TCCL_D void pull_finish(PullState& st, const PullArgs& a, int num_wgs) const {
+    if (a.peers == 0) return;
+    wait_vmem();
+    if (st.pending_lp >= 0) pull_store_pending(st, a, st.pending_lds);
+    st.probe_group = -1;
+    const int64_t deadline = now_ticks() + a.spin_ticks;
+    bool ok = true;
+    constexpr int kBatch = 4;
+    while (ok && st.next_slot < a.peers) {
+      pull_select(st, a, st.next_slot);
+      u32x4 v[kBatch];
+      uint32_t off[kBatch];
+      bool valid[kBatch];
+      int n = 0;
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        valid[k] = false;
+        const int lp = st.next_lp + k * st.stride;
+        if (ok && lp < a.pieces) {
+          ok = pull_wait_ready(st, a, pull_last_unit(a, lp), deadline);
+          if (ok) {
+            off[k] = pull_offset(a, lp, valid[k]);
+            v[k] = ld16<kCoherent>(window(st.src_base), off[k]);
+            n = k + 1;
+          }
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k)
+        if (valid[k]) st16<kStreaming>(window(st.dst_base), off[k], v[k]);
+      st.next_lp += n * st.stride;
+      if (n < kBatch) {  // the block is finished (or a wait gave up)
+        st.next_lp -= a.pieces;
+        if (st.next_lp < 0) st.next_lp = 0;  // only after a failed wait
+        ++st.next_slot;
+        pull_normalise(st, a);
+      }
+    }
+    if (!ok && lane == 0 && a.fault) *a.fault = 1;
+    wait_vmem();
+    __syncthreads();
+    // One arrival per workgroup on barrier[0]; the last one to arrive brings the other groups'
+    // words up to the same count (concurrent adds to one word cost ~7 ns each on this part).
+    if (tid == 0 && a.barrier) {
+      const int32_t prev = tile_signal_add<true>(a.barrier, 0, 1);
+      if (prev + 1 == a.epoch * num_wgs) {
+        for (int g = 0; g < a.n_groups; ++g) {
+          if (g > 0) tile_signal_add<true>(a.barrier, g, num_wgs);
+          if (a.trace_done_clock) a.trace_done_clock[g] = now_ticks();
+        }
+      }
+    }
+  }
+
+  // One K step: the MFMAs of this step run from `cur` while the next step's operands
+  // stream into `nxt`, one A piece and one B piece per k-chunk.  Fragments are single
+  // buffered: two waves share a SIMD, so while one waits for its LDS reads the other issues
+  // MFMAs; holding a second fragment set would push the kernel past 256 registers and the
+  // spill reloads would drain the load queue every step.  The scheduling barrier keeps the
+  // compiler from hoisting the next chunk's reads across the MFMAs.
+  TCCL_D void k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
+                     PullState& pull, char* pull_load, const char* pull_store) const {
+    pull_step(pull, pa, pull_load, pull_store);
+#pragma unroll
+    for (int kk = 0; kk < kBK / 16; ++kk) {
+      Vec fa[4], fb[2];
+      load_frags(cur, rd, kk, fa, fb);
+      issue_piece(nxt, src, kt_load, kk);
+#pragma unroll
+      for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = Mfma<InT>::run(fb[bj], fa[bi], acc[bi][bj]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  template <int kPolicy>
+  TCCL_D void epilogue(int row0, int col0, const f32x16 (&acc)[4][2]) const {
+    constexpr int kEsz = sizeof(OutT);
+    constexpr int kRowBytes = 64 * kEsz;
+    constexpr int kChunks = kRowBytes / 16;
+    constexpr int kPerChunk = 16 / kEsz;
+    char* win = lds + wave * (32 * 64 * 4);  // 8 KiB per wave, 64 KiB in all: inside stage 0
+    const int half = lane >> 5, l32 = lane & 31;
+    OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
+    const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
+    PushArgs push;
+    push.n = 0;
+    if (push_offset >= 0) push = late_kernarg<PushArgs>(push_offset);
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi) {
+      __syncthreads();
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n_local = bj * 32 + 8 * q + 4 * half;
+          OutT v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[bi][bj][4 * q + e] * g.alpha);
+          const int byte = n_local * kEsz;
+          const int chunk = (byte >> 4) ^ (l32 & 7);
+          char* p = win + l32 * kRowBytes + chunk * 16 + (byte & 15);
+          if constexpr (kEsz == 2) {
+            uint2 u;
+            __builtin_memcpy(&u, v, 8);
+            *(uint2*)p = u;
+          } else {
+            u32x4 u;
+            __builtin_memcpy(&u, v, 16);
+            *(u32x4*)p = u;
+          }
+        }
+      __syncthreads();
+      constexpr int kRounds = (32 * kChunks) / 64;
+      u32x4 v[kRounds];
+      int lrow[kRounds], lcol[kRounds];
+      bool live[kRounds];
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) {
+        const int idx = lane + 64 * r;
+        const int row = idx / kChunks, chunk = idx % kChunks;
+        v[r] = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
+        lrow[r] = wm * 128 + bi * 32 + row;
+        lcol[r] = wn * 64 + chunk * kPerChunk;
+        live[r] = row0 + lrow[r] < g.M && col0 + lcol[r] < g.N;
+        if (live[r]) __builtin_amdgcn_raw_buffer_store_b128(v[r], rc, (uint32_t)((lrow[r] * g.ldc + lcol[r]) * kEsz), 0, kPolicy);
+      }
+      for (int t = 0; t < push.n; ++t) {
+        char* base = push.base[t] + ((int64_t)row0 * push.ld + col0 + push.col_shift) * kEsz;
+        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffffu, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+          const int col = col0 + lcol[r];
+          if (live[r] && col >= push.col_lo && col < push.col_hi)
+            __builtin_amdgcn_raw_buffer_store_b128(v[r], rt, (uint32_t)((lrow[r] * push.ld + lcol[r]) * kEsz), 0, kCoherent);
+        }
+      }
+    }
+  }
+
+  template <int kPolicy>
+  TCCL_D void macro_tile(int row0, int col0, PullState& pull) const {
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const Source src = make_source(row0, col0);
+    const Reader rd = make_reader();
+    // K steps are taken in pairs so that each call names its two stages statically and the
+    // accumulators flow through one straight loop body.  An odd step count is rounded up: the
+    // extra step (like the final look-ahead load) lies wholly past K and reads zeros.
+    const int ksteps = ((g.K + kBK - 1) / kBK + 1) & ~1;
+    __syncthreads();  // the previous tile's epilogue has left LDS
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
+    wait_vmem();
+    __syncthreads();
+    for (int kt = 0; kt < ksteps; kt += 2) {
+      k_step(lds, lds1, src, rd, kt + 1, acc, pull, bg0, bg1);
+      wait_vmem();
+      __syncthreads();
+      k_step(lds1, lds, src, rd, kt + 2, acc, pull, bg1, bg0);
+      wait_vmem();
+      __syncthreads();
+    }
+    epilogue<kPolicy>(row0, col0, acc);
+  }
+
+  // Publish every plan tile the macro tile (mm, mn) covers.
+  // Plan tiles of one row share a TileGroup, so the group counts are summed up here and
+  // each group gets one add (concurrent adds to one word serialise).
+  TCCL_D void publish(const SignalArgs& s, int mm, int mn) const {
+    const int tm0 = mm * (kMacro / g.block_m), tn0 = mn * (kMacro / g.block_n);
+    int group = -1, count = 0;
+    for (int dm = 0; dm < kMacro / g.block_m; ++dm)
+      for (int dn = 0; dn < kMacro / g.block_n; ++dn) {
+        const int tm = tm0 + dm, tn = tn0 + dn;
+        if (tm >= g.tile_rows || tn >= g.tile_cols) continue;
+        const int tile_id = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
+        if (s.mode == kSignalTile) {
+          tile_signal<true>(s.locks, tile_id);
+          continue;
+        }
+        const int gi = s.group_table[tile_id];
+        if (gi != group && count > 0) {
+          tile_signal_add<true>(s.counter, group, count);
+          count = 0;
+        }
+        group = gi;
+        ++count;
+      }
+    if (count > 0) tile_signal_add<true>(s.counter, group, count);
+  }
+
+  TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
+    const int total = m.rows * m.cols;
+    PullState pull = pull_begin(pa, wg, num_wgs);
+    pull_prime(pull, pa, bg1);
+    for (int slot = wg; slot < total; slot += num_wgs) {
+      const int id = tile_for_slot(slot, total, m.xcds, m.span);
+      const TileCoord c = macro_coords(id, m);
+      const int row0 = c.m * kMacro, col0 = c.n * kMacro;
+      if (s.mode == kSignalNone && push_offset < 0) {
+        macro_tile<0>(row0, col0, pull);
+      } else {
+        macro_tile<kCoherent>(row0, col0, pull);
+        wait_vmem();
+        __syncthreads();
+        if (tid == 0 && s.mode != kSignalNone) publish(s, c.m, c.n);
+      }
+    }
+    pull_finish(pull, pa, num_wgs);
+  }
+};
+#endif  // __HIP_DEVICE_COMPILE__
+
+}  // namespace tccl

@@ -60,6 +60,7 @@ class _FusedBase:
         transport: P2PTransportPlan | None = None,
         num_comm_wgs: int = 0,
         num_gemm_wgs: int = 0,
+        macro_tile: int = 0,
         trace: bool = False,
         spin_limit_ns: int = _launch.DEFAULT_SPIN_LIMIT_NS,
     ) -> None:
@@ -70,6 +71,7 @@ class _FusedBase:
         self.tau_min_bytes, self.max_groups = tau_min_bytes, max_groups
         self.transport = transport or build_p2p_transport_plan(comm_mode="push", copy_elems=16384)
         self.num_comm_wgs, self.num_gemm_wgs = num_comm_wgs, num_gemm_wgs
+        self.macro_tile = macro_tile
         self.trace = trace
         self.spin_limit_ns = spin_limit_ns
         self.spec: CollectiveSpec | None = None
@@ -177,7 +179,7 @@ class FusedGemmAllGather(_FusedBase):
     def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0) -> torch.Tensor:
         gemm = _launch.gemm_desc(
             A, B, self.local_block, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
-            alpha=alpha, num_wgs=self.num_gemm_wgs,
+            alpha=alpha, num_wgs=self.num_gemm_wgs, macro_tile=self.macro_tile,
         )
         view, transport, sync = self._descs(self.directions, variant)
         rc = _lib.load().tccl_gemm_allgather(
@@ -221,7 +223,7 @@ class FusedGemmReduceScatter(_FusedBase):
     def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0) -> torch.Tensor:
         gemm = _launch.gemm_desc(
             A, B, self.partial, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
-            alpha=alpha, num_wgs=self.num_gemm_wgs,
+            alpha=alpha, num_wgs=self.num_gemm_wgs, macro_tile=self.macro_tile,
         )
         view, transport, sync = self._descs(_lib.DIR_PULL, variant)
         rc = _lib.load().tccl_gemm_reducescatter(
