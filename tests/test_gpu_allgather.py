@@ -13,6 +13,9 @@ from tests.gpu_util import assert_gemm_close, bits, into_heap, seeded
 pytestmark = pytest.mark.gpu
 
 VARIANTS = ["s0", "s1", "s2"]
+# 128: one launch whose workgroups split into a GEMM role and a communication role.
+# 256: large-tile launch; pushes leave from the GEMM epilogue, S2 pulls run inside the K loop.
+MACRO = [128, 256]
 
 
 def make(world, M, N, dtype=torch.float16, heap_bytes=256 << 20, **kw):
@@ -37,9 +40,10 @@ def fill_peer_blocks(ops, M, N, dtype, seed=2):
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("directions", ["both", "push", "pull"])
-def test_small_two_ranks_against_oracle(lib, variant, directions):
+@pytest.mark.parametrize("macro", MACRO)
+def test_small_two_ranks_against_oracle(lib, variant, directions, macro):
     M, N, K = 512, 512, 256
-    heaps, ops = make(2, M, N, directions=directions)
+    heaps, ops = make(2, M, N, directions=directions, macro_tile=macro)
     try:
         op = ops[0]
         A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
@@ -72,10 +76,11 @@ def test_small_two_ranks_against_oracle(lib, variant, directions):
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-def test_ragged_shape_four_ranks_many_groups(lib, variant):
+@pytest.mark.parametrize("macro", MACRO)
+def test_ragged_shape_four_ranks_many_groups(lib, variant, macro):
     """M not a multiple of the tile, several groups per rank, fan-out to three peers."""
     M, N, K = 1000, 264, 72
-    heaps, ops = make(4, M, N, dtype=torch.bfloat16, tau_min_bytes=1, group_m=2,
+    heaps, ops = make(4, M, N, dtype=torch.bfloat16, tau_min_bytes=1, group_m=2, macro_tile=macro,
                       transport=__import__("tileccl_amd.v2", fromlist=["x"]).build_p2p_transport_plan(
                           comm_mode="push", copy_elems=1024))
     try:
@@ -141,6 +146,36 @@ def test_baseline_configs_1_and_2_properties(lib, local_M, block_m):
         normal = base.abs() >= 2.0**-13
         assert torch.equal(doubled[normal], 2 * base[normal])
         assert (doubled - 2 * base).abs().max().item() <= 2.0**-23
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+def test_pull_with_padded_rows_and_short_k(lib):
+    """Large-tile S2 with fewer K steps than pieces per wavefront (the rest of the pull runs
+    after the last tile) and a gathered buffer whose rows are not contiguous."""
+    from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+    M, N, K = 768, 520, 64
+    heaps = SymmetricHeap.create_all(64 << 20, 3)
+    try:
+        ops = [FusedGemmAllGather(h, M, N, torch.float16, directions="both", macro_tile=256, tau_min_bytes=1, group_m=1)
+               for h in heaps]
+        op = ops[0]
+        assert op.plan.n_groups > 1
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        blocks = fill_peer_blocks(ops, M, N, torch.float16)
+        for variant in VARIANTS:
+            op.out.zero_()
+            op.mark_peers_ready()
+            op(A, B, variant)
+            op.check_faults()
+            mine = op.out[:M].clone()
+            assert_gemm_close(mine, A_cpu.float() @ B_cpu.float(), tight=0.004)
+            for p in (1, 2):
+                assert torch.equal(bits(op.peer_out(p)[:M]), bits(mine)), (variant, p)
+                assert torch.equal(bits(op.out[p * M:(p + 1) * M]).cpu(), bits(blocks[p])), (variant, p)
     finally:
         for h in heaps:
             h.cleanup()

@@ -37,12 +37,17 @@ SHAPES = [
 ]
 
 
+# macro_tile: 128 = the 128 x 128 kernel, 256 = the large-tile kernel (0 would pick by size)
+MACRO = [128, 256]
+
+
 @pytest.mark.parametrize("M,N,K", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_gemm_matches_fp32_matmul(lib, M, N, K, dtype):
+@pytest.mark.parametrize("macro", MACRO)
+def test_gemm_matches_fp32_matmul(lib, M, N, K, dtype, macro):
     A = seeded((M, K), 0, dtype)
     B = seeded((K, N), 1, dtype, scale=K**-0.5)
-    got = run_gemm(lib, A, B, dtype)
+    got = run_gemm(lib, A, B, dtype, macro_tile=macro)
     ref32 = A.float() @ B.float()
     assert not torch.isnan(got.float()).any()
     # one rounding of an O(1) value: half an ulp of fp16 (2^-11 rel.) / bf16 (2^-8 rel.) at |x| < 8
@@ -54,37 +59,43 @@ def test_gemm_matches_fp32_matmul(lib, M, N, K, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_fp32_output_keeps_the_accumulator(lib, dtype):
+@pytest.mark.parametrize("macro", MACRO)
+def test_fp32_output_keeps_the_accumulator(lib, dtype, macro):
     A, B = seeded((384, 256), 3, dtype), seeded((256, 640), 4, dtype, scale=1 / 16)
-    got = run_gemm(lib, A, B, torch.float32)
+    got = run_gemm(lib, A, B, torch.float32, macro_tile=macro)
     ref32 = A.float() @ B.float()
     assert (got.cpu() - ref32).abs().max().item() < 1e-4  # only the fp32 summation order differs
 
 
-def test_alpha_and_plan_tile_256(lib):
+@pytest.mark.parametrize("macro", MACRO)
+def test_alpha_and_plan_tile_256(lib, macro):
     A, B = seeded((512, 128), 5), seeded((128, 384), 6, scale=128**-0.5)
     ref32 = 0.5 * (A.float() @ B.float())
-    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5), ref32, tight=0.004)
-    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, group_m=3), ref32, tight=0.004)
-    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, block_n=256, num_wgs=7), ref32, tight=0.004)
+    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, macro_tile=macro), ref32, tight=0.004)
+    assert_gemm_close(run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, group_m=3, macro_tile=macro), ref32, tight=0.004)
+    assert_gemm_close(
+        run_gemm(lib, A, B, torch.float16, alpha=0.5, block_m=256, block_n=256, num_wgs=7, macro_tile=macro), ref32, tight=0.004
+    )
 
 
-def test_exact_small_integers(lib):
+@pytest.mark.parametrize("macro", MACRO)
+def test_exact_small_integers(lib, macro):
     """Integer-valued inputs whose products and sums are exact in fp16/fp32: bit-exact result."""
     g = torch.Generator().manual_seed(7)
     A = torch.randint(-3, 4, (256, 192), generator=g).half()
     B = torch.randint(-3, 4, (192, 256), generator=g).half()
-    got = run_gemm(lib, A, B, torch.float16)
+    got = run_gemm(lib, A, B, torch.float16, macro_tile=macro)
     assert torch.equal(got.cpu(), (A.float() @ B.float()).half())
 
 
-def test_rows_beyond_M_and_cols_beyond_N_are_untouched(lib):
+@pytest.mark.parametrize("macro", MACRO)
+def test_rows_beyond_M_and_cols_beyond_N_are_untouched(lib, macro):
     from tileccl_amd import _launch, _lib
 
     A, B = seeded((100, 64), 8).cuda(), seeded((64, 72), 9).cuda()
     backing = torch.full((128, 128), 7.0, dtype=torch.float16, device="cuda")
     out = backing[:100, :72]  # ldc = 128
-    desc = _launch.gemm_desc(A, B, out)
+    desc = _launch.gemm_desc(A, B, out, macro_tile=macro)
     _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
     torch.cuda.synchronize()
     assert torch.all(backing[100:] == 7.0) and torch.all(backing[:, 72:] == 7.0)
@@ -106,6 +117,9 @@ def test_unsupported_layouts_fail_loudly(lib):
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
     with pytest.raises(ValueError, match="must be a multiple of 128x128"):
         d = _launch.gemm_desc(A, B, out, block_m=64)
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="macro_tile=64 must be 0, 128 or 256"):
+        d = _launch.gemm_desc(A, B, out, macro_tile=64)
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
     with pytest.raises(ValueError, match="no kernel for in_dtype"):
         d = _launch.gemm_desc(A, B, torch.empty(128, 128, dtype=torch.bfloat16, device="cuda"))

@@ -25,10 +25,11 @@ def make(world, M, N, heap_bytes=256 << 20, **kw):
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("partial_dtype,out_dtype", [(torch.float32, torch.float16), (torch.bfloat16, torch.bfloat16),
                                                     (torch.float32, torch.bfloat16)])
-def test_small_two_ranks_bit_exact(lib, variant, partial_dtype, out_dtype):
+@pytest.mark.parametrize("macro", [128, 256])
+def test_small_two_ranks_bit_exact(lib, variant, partial_dtype, out_dtype, macro):
     M, N, K = 512, 512, 256
     in_dtype = torch.bfloat16 if partial_dtype == torch.bfloat16 else torch.float16
-    heaps, ops = make(2, M, N, partial_dtype=partial_dtype, out_dtype=out_dtype)
+    heaps, ops = make(2, M, N, partial_dtype=partial_dtype, out_dtype=out_dtype, macro_tile=macro)
     try:
         op = ops[0]
         assert op.plan.groups == [(0, 256, 8), (256, 512, 8)]  # one wave, cut at the owner border

@@ -51,7 +51,8 @@ def test_translate_ptr_host(heap):
     assert ipc.translate_ptr(ipc.translate_ptr(t.data_ptr(), 0, 1, bases), 1, 0, bases) == t.data_ptr()
 
 
-def test_fused_launch_times_out_cleanly_when_a_peer_never_signals(lib):
+@pytest.mark.parametrize("macro", [128, 256])
+def test_fused_launch_times_out_cleanly_when_a_peer_never_signals(lib, macro):
     """Pull from a peer whose counters stay at zero: every communication workgroup gives up
     after the (tiny, host-set) spin limit, the kernel ends normally and the host raises."""
     from tests.gpu_util import into_heap, seeded
@@ -59,7 +60,8 @@ def test_fused_launch_times_out_cleanly_when_a_peer_never_signals(lib):
 
     heaps = SymmetricHeap.create_all(64 << 20, 2)
     try:
-        op = FusedGemmAllGather(heaps[0], 256, 256, torch.float16, directions="pull", spin_limit_ns=200_000)
+        op = FusedGemmAllGather(heaps[0], 256, 256, torch.float16, directions="pull", spin_limit_ns=200_000,
+                                macro_tile=macro)
         FusedGemmAllGather(heaps[1], 256, 256, torch.float16)  # same allocation sequence on the peer
         A, B = into_heap(heaps[0], seeded((256, 64), 0)), into_heap(heaps[0], seeded((64, 256), 1))
         op(A, B, "s2")
