@@ -117,12 +117,16 @@ TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
 // registers (and spill into vector registers) all through the K loop.  The empty asm hides
 // the address from the optimiser until control reaches this point.
 template <typename T>
-TCCL_D T late_kernarg(int offset) {
+TCCL_D const __attribute__((address_space(4))) T* late_kernarg_ptr(int offset) {
   typedef const __attribute__((address_space(4))) char* KernargPtr;
   KernargPtr p = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr() + offset;
   asm volatile("" : "+s"(p));
+  return (const __attribute__((address_space(4))) T*)p;
+}
+template <typename T>
+TCCL_D T late_kernarg(int offset) {
   T v;
-  __builtin_memcpy(&v, p, sizeof(T));
+  __builtin_memcpy(&v, late_kernarg_ptr<T>(offset), sizeof(T));
   return v;
 }
 
@@ -472,9 +476,10 @@ struct Gemm256 {
     const int half = lane >> 5, l32 = lane & 31;
     OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
     const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
-    PushArgs push;
-    push.n = 0;
-    if (push_offset >= 0) push = late_kernarg<PushArgs>(push_offset);
+    // Fields are read through the argument block itself: a local copy of base[] would be
+    // indexed dynamically and end up in scratch memory.
+    const auto* push = late_kernarg_ptr<PushArgs>(push_offset < 0 ? 0 : push_offset);
+    const int push_n = push_offset >= 0 ? push->n : 0;
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
       __syncthreads();
@@ -514,14 +519,16 @@ struct Gemm256 {
         live[r] = row0 + lrow[r] < g.M && col0 + lcol[r] < g.N;
         if (live[r]) __builtin_amdgcn_raw_buffer_store_b128(v[r], rc, (uint32_t)((lrow[r] * g.ldc + lcol[r]) * kEsz), 0, kPolicy);
       }
-      for (int t = 0; t < push.n; ++t) {
-        char* base = push.base[t] + ((int64_t)row0 * push.ld + col0 + push.col_shift) * kEsz;
+      for (int t = 0; t < push_n; ++t) {
+        const int64_t push_ld = push->ld;
+        const int col_lo = push->col_lo, col_hi = push->col_hi;
+        char* base = push->base[t] + ((int64_t)row0 * push_ld + col0 + push->col_shift) * kEsz;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffffu, 0x00020000);
 #pragma unroll
         for (int r = 0; r < kRounds; ++r) {
           const int col = col0 + lcol[r];
-          if (live[r] && col >= push.col_lo && col < push.col_hi)
-            __builtin_amdgcn_raw_buffer_store_b128(v[r], rt, (uint32_t)((lrow[r] * push.ld + lcol[r]) * kEsz), 0, kCoherent);
+          if (live[r] && col >= col_lo && col < col_hi)
+            __builtin_amdgcn_raw_buffer_store_b128(v[r], rt, (uint32_t)((lrow[r] * push_ld + lcol[r]) * kEsz), 0, kCoherent);
         }
       }
     }
