@@ -177,13 +177,15 @@ TCCL_D u32x4 pack8<__bf16>(const float (&f)[8]) {
   return __builtin_bit_cast(u32x4, h);
 }
 
-constexpr int kReduceUnroll = 2;
 
 // Sum order: the owner's addend first, then the other ranks in ascending order
 // (tile_reduce_scatter: local chunk, then peers ascending; collectives.py:766-781).
 template <typename PT, typename OT, int kPolicy, int kThreads>
 TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   constexpr uint32_t kSrcUnit = 8 * sizeof(PT);
+  // Units a thread keeps in flight.  A 512-thread workgroup has its CU to itself (the tail of
+  // the large-tile kernel), so it must carry the loads that several small workgroups would.
+  constexpr int kReduceUnroll = kThreads >= 512 ? 4 : 2;
   const int tid = threadIdx.x;
   const int dst_rank = __builtin_ctz(x.dst_ranks);
   const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[dst_rank] + x.dst_off);
