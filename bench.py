@@ -24,6 +24,10 @@ if str(ROOT) not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0}
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
+# this script scaled by what the same counters read for the bulk copy kernel of known size
+# (profiles/fused256_kernel_c1_s2_counters.md).  Known only for the default configuration.
+MEASURED_TRAFFIC_BYTES = {("c1", "s2", 0): int(175.8 * 2**20)}
 
 WORKLOADS = {
     # name: (local M, N, K, block_m)
@@ -184,7 +188,7 @@ def main() -> int:
             "peak": PEAK_TFLOPS["f16"],
             "unit": "TFLOP/s",
             "frac": round(tflops / PEAK_TFLOPS["f16"], 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.variant, args.macro_tile)),
             "kernel_ms": round(chosen["event_ms_mean"], 5),
         },
     }
