@@ -1,0 +1,107 @@
+"""fp8 (OCP e4m3) GEMM and GEMM -> ReduceScatter on gfx950's 32x32x64 fp8 MFMA.
+
+Inputs follow the BASELINE fp8 recipe: N(0,1) samples divided by a per-tensor fp32 scale,
+clipped to +-448 and rounded to e4m3; the scales' product multiplies the accumulator.
+Products of two e4m3 values are exact in fp32, so the GPU result differs from the oracle
+(dequantise, fp32 matmul) only by fp32 summation order and the output rounding; the stated
+tolerance for fp8 is rtol 5e-2, and a tight absolute bound rules out layout mistakes."""
+
+import ctypes as C
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import assert_gemm_close, bits, into_heap, seeded
+
+pytestmark = pytest.mark.gpu
+
+F8 = torch.float8_e4m3fn
+
+
+def quantise(shape, seed, std=1.0):
+    """(e4m3 tensor, dequantisation scale) for x ~ N(0, std^2): stored value = clip(x / scale, +-448),
+    with the scale chosen so that one standard deviation is stored as 64."""
+    x = seeded(shape, seed, torch.float32, scale=std)
+    scale = std / 64
+    return (x / scale).clamp(-448.0, 448.0).to(F8), scale
+
+
+def run_gemm(lib, A_cpu, B_cpu, out_dtype, alpha=1.0, **kw):
+    from tileccl_amd import _launch, _lib
+
+    A, B = A_cpu.cuda(), B_cpu.cuda()
+    out = torch.full((A.shape[0], B.shape[1]), float("nan"), dtype=out_dtype, device="cuda")
+    desc = _launch.gemm_desc(A, B, out, alpha=alpha, **kw)
+    _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 256, 64), (512, 768, 512), (300, 272, 80), (1, 16, 16),
+                                   (1024, 4096, 1024)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_fp8_gemm_matches_dequantised_matmul(lib, M, N, K, out_dtype):
+    A, sa = quantise((M, K), 0)
+    B, sb = quantise((K, N), 1, K**-0.5)
+    got = run_gemm(lib, A, B, out_dtype, alpha=sa * sb)
+    ref32 = (A.float() @ B.float()) * (sa * sb)
+    assert not torch.isnan(got.float()).any()
+    tight = {torch.float32: 1e-3, torch.float16: 0.004, torch.bfloat16: 0.032}[out_dtype]
+    assert_gemm_close(got, ref32, rtol=5e-2, atol=1e-1, tight=tight)
+    want = oracle.gemm(A, B, out_dtype, alpha=sa * sb)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= tight
+
+
+def test_fp8_exact_small_integers(lib):
+    """Integer-valued e4m3 inputs: every product and partial sum is exact, so is the result."""
+    g = torch.Generator().manual_seed(7)
+    A = torch.randint(-3, 4, (256, 320), generator=g).float().to(F8)
+    B = torch.randint(-3, 4, (320, 512), generator=g).float().to(F8)
+    got = run_gemm(lib, A, B, torch.float32)
+    assert torch.equal(got.cpu(), A.float() @ B.float())
+
+
+def test_fp8_needs_the_large_tile_kernel(lib):
+    from tileccl_amd import _launch, _lib
+
+    A, B = torch.zeros(256, 64, dtype=F8, device="cuda"), torch.zeros(64, 256, dtype=F8, device="cuda")
+    out = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="fp8 inputs need the 256x256 kernel"):
+        d = _launch.gemm_desc(A, B, out, macro_tile=128)
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="K=72 must be a multiple of 16"):
+        d = _launch.gemm_desc(torch.zeros(256, 72, dtype=F8, device="cuda"), torch.zeros(72, 256, dtype=F8, device="cuda"), out)
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+
+
+@pytest.mark.parametrize("variant", ["s0", "s1", "s2"])
+def test_fp8_reduce_scatter_two_ranks(lib, variant):
+    """The fp8 ReduceScatter configuration at a small size: bf16 partial, resident bf16 peer
+    partial, fp32 reduction, bf16 output; the reduction is bit-exact against the oracle run
+    on the partial the GPU produced."""
+    from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
+
+    M, N, K = 1024, 512, 256
+    heaps = SymmetricHeap.create_all(64 << 20, 2)
+    try:
+        ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=torch.bfloat16, out_dtype=torch.bfloat16) for h in heaps]
+        op = ops[0]
+        A_cpu, sa = quantise((M, K), 0)
+        B_cpu, sb = quantise((K, N), 1, K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        peer = seeded((M, N), 2, torch.bfloat16)
+        ops[1].partial.copy_(peer)
+        for o in ops:
+            o.out.zero_()
+        op.mark_peers_ready()
+        op(A, B, variant, scale_a=sa, scale_b=sb)
+        op.check_faults()
+        assert_gemm_close(op.partial, (A_cpu.float() @ B_cpu.float()) * (sa * sb), rtol=5e-2, tight=0.032)
+        partials = [op.partial.cpu(), peer]
+        for owner in (0, 1):
+            want = oracle.reduce_rows(partials, owner, torch.bfloat16)
+            assert torch.equal(bits(ops[owner].out).cpu(), bits(want)), f"owner {owner}"
+    finally:
+        for h in heaps:
+            h.cleanup()

@@ -163,6 +163,10 @@ __global__ void prim_wait_ge_kernel(int32_t* w, int i, int thr, int64_t ticks, i
 // ------------------------------------------------------------------------------------------
 constexpr int64_t kDefaultSpinNs = 2000000000ll;
 
+bool plan_tile_fits_macro(const tccl_gemm_desc* d) {
+  return (d->block_m == 128 || d->block_m == 256) && (d->block_n == 128 || d->block_n == 256);
+}
+
 int check_gemm(const tccl_gemm_desc* d) {
   if (!d) return fail(TCCL_ERR_INVALID, "gemm descriptor is NULL");
   if (!d->A || !d->B || !d->C) return fail(TCCL_ERR_INVALID, "gemm: A, B and C must be non-NULL");
@@ -175,6 +179,8 @@ int check_gemm(const tccl_gemm_desc* d) {
   const size_t isz = dtype_size(d->in_dtype), osz = dtype_size(d->out_dtype);
   if (!isz || !osz) return fail(TCCL_ERR_INVALID, "gemm: unknown dtype");
   if (d->in_dtype == TCCL_F32) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp32 inputs have no MFMA kernel here");
+  if (d->in_dtype == TCCL_F8E4M3 && (d->macro_tile == 128 || !plan_tile_fits_macro(d)))
+    return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 inputs need the 256x256 kernel (macro_tile 0 or 256, plan tile edges 128 or 256)");
   if (d->out_dtype == TCCL_F8E4M3) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 output is not supported");
   const int in_vec = (int)(16 / isz), out_vec = (int)(16 / osz);
   if (d->K % in_vec) return fail(TCCL_ERR_UNSUPPORTED, "gemm: K=%d must be a multiple of %d", d->K, in_vec);
@@ -311,13 +317,11 @@ int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tcc
 }
 
 // ---- large-tile path ----------------------------------------------------------------------------
-bool plan_tile_fits_macro(const tccl_gemm_desc* d) {
-  return (d->block_m == 128 || d->block_m == 256) && (d->block_n == 128 || d->block_n == 256);
-}
 
 // 256 x 256 tiles pay off once there are enough of them to occupy most CUs; below that
 // the 128 x 128 kernel spreads the work over more workgroups.
 bool use_macro(const tccl_gemm_desc* d, const tccl_device_info& dev) {
+  if (d->in_dtype == TCCL_F8E4M3) return true;  // fp8 exists only as the large-tile kernel (check_gemm vets the plan tile)
   if (!plan_tile_fits_macro(d)) return false;
   if (d->macro_tile == 128) return false;
   if (d->macro_tile == 256) return true;
@@ -360,6 +364,9 @@ int launch_gemm256(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const t
   if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_gemm256_t<_Float16, float>(g, m, wgs, stream);
   if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_gemm256_t<__bf16, __bf16>(g, m, wgs, stream);
   if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_gemm256_t<__bf16, float>(g, m, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_BF16) return launch_gemm256_t<tccl::fp8e4m3, __bf16>(g, m, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F16) return launch_gemm256_t<tccl::fp8e4m3, _Float16>(g, m, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F32) return launch_gemm256_t<tccl::fp8e4m3, float>(g, m, wgs, stream);
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 
@@ -375,6 +382,9 @@ int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
   if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused256_t<_Float16, float>(f, wgs, stream);
   if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused256_t<__bf16, __bf16>(f, wgs, stream);
   if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused256_t<__bf16, float>(f, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_BF16) return launch_fused256_t<tccl::fp8e4m3, __bf16>(f, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F16) return launch_fused256_t<tccl::fp8e4m3, _Float16>(f, wgs, stream);
+  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F32) return launch_fused256_t<tccl::fp8e4m3, float>(f, wgs, stream);
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 

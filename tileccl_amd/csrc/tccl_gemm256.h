@@ -35,12 +35,25 @@
 
 namespace tccl {
 
+// OCP fp8 e4m3 ("e4m3fn"), the 8-bit input type of gfx950's v_mfma_f32_32x32x64_f8f6f4.
+struct fp8e4m3 {
+  uint8_t bits;
+};
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+#if defined(__HIP_DEVICE_COMPILE__)
+template <>
+struct Mfma<fp8e4m3> {
+  typedef i32x8 Vec;  // 32 consecutive k of one row / column
+  // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled form.
+  static TCCL_D f32x16 run(Vec a, Vec b, f32x16 c) { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0); }
+};
+#endif
+
 constexpr int kMacro = 256;
 constexpr int kThreads256 = 512;
 constexpr int kARow256 = 128;                              // A: bytes per row of one stage (64 k)
 constexpr int kAStage256 = kMacro * kARow256;              // 32 768 B
-constexpr int kBPitch256 = 512;                            // B: bytes per k row (256 columns)
-constexpr int kBStage256 = kBK * kBPitch256;               // 32 768 B
+constexpr int kBStage256 = 32768;                          // B: (128 / element size) k rows of 256 columns
 constexpr int kStage256 = kAStage256 + kBStage256;         // A then B
 constexpr int kLds256 = 2 * kStage256;                     // two stages: 131 072 B (two arrays)
 
@@ -133,6 +146,12 @@ TCCL_D T late_kernarg(int offset) {
 template <typename InT, typename OutT>
 struct Gemm256 {
   typedef typename Mfma<InT>::Vec Vec;
+  static constexpr int kEszIn = sizeof(InT);
+  static constexpr int kStepK = kARow256 / kEszIn;     // K per step: 64 (16-bit), 128 (fp8)
+  static constexpr int kChunkK = 16 / kEszIn;          // elements per 16-byte chunk
+  static constexpr int kBPitch = kMacro * kEszIn;      // bytes per k row of the B stage
+  static constexpr int kBRowsPerPiece = 1024 / kBPitch;  // k rows one 1 KiB load covers: 2 or 4
+  static constexpr bool kFp8 = kEszIn == 1;
 
   const GemmArgs& g;
   const PullArgs& pa;
@@ -158,7 +177,8 @@ struct Gemm256 {
   // Where this lane's four A pieces and four B pieces of a K step come from (byte offsets
   // into the buffer resources at K step 0).  Piece i of wave w fills
   //   A rows 8*(4w+i) .. +7      (lane l: row + l/8, slot l%8)
-  //   B k rows 2*(4w+i), +1      (lane l: k row + l/32, slot l%32)
+  //   B k rows 2*(4w+i), +1      (lane l: k row + l/32, slot l%32)            16-bit inputs
+  //   B k rows 4*(4w+i) .. +3    (lane l: k row + l/16, slot l%16)            fp8 inputs
   struct Source {
     __amdgpu_buffer_rsrc_t a, b;
     uint32_t off_a[4], off_b[4];
@@ -179,12 +199,18 @@ struct Gemm256 {
       const int row = 8 * (4 * wave + i) + (lane >> 3);
       const int kc = (lane & 7) ^ ((row >> 1) & 7);
       s.off_a[i] = (uint32_t)(row * g.lda * kEsz + kc * 16);
-      const int k = 2 * (4 * wave + i) + (lane >> 5);
-      const int c = (lane & 31) ^ (4 * (k & 3));
-      s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
+      if constexpr (kFp8) {
+        const int k = 4 * (4 * wave + i) + (lane >> 4);
+        const int c = (lane & 15) ^ (2 * (k & 7));
+        s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
+      } else {
+        const int k = 2 * (4 * wave + i) + (lane >> 5);
+        const int c = (lane & 31) ^ (4 * (k & 3));
+        s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
+      }
     }
-    s.step_a = kBK * kEsz;
-    s.step_b = (uint32_t)(kBK * g.ldb * kEsz);
+    s.step_a = kStepK * kEsz;
+    s.step_b = (uint32_t)(kStepK * g.ldb * kEsz);
     return s;
   }
 
@@ -192,10 +218,10 @@ struct Gemm256 {
   // end of the buffer so that they read as zero (B rows >= K already lie past it).
   TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
     const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);  // as in make_source
-    const bool dead = kt * kBK + kc * 8 >= g.K;
+    const bool dead = kt * kStepK + kc * kChunkK >= g.K;
     const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + kt * s.step_a;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + 8 * (4 * wave + i) * kARow256), 16, oa, 0, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + 2 * (4 * wave + i) * kBPitch256), 16,
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + (4 * wave + i) * 1024), 16,
                                              s.off_b[i] + kt * s.step_b, 0, 0, 0);
   }
 
@@ -212,9 +238,45 @@ struct Gemm256 {
     Reader r;
     r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
     r.a_swz = (uint32_t)((l32 >> 1) & 7);
-    const int chunk = (wn * 8 + grp * 2 + (cq >> 1)) ^ (4 * t);
-    r.b_base0 = (uint32_t)(kAStage256 + (8 * half + t) * kBPitch256 + chunk * 16 + (cq & 1) * 8);
+    if constexpr (kFp8) {
+      // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns of k row i/2
+      // (column block i%2) and lane j receives 8 consecutive k of column j.  Four reads
+      // (k + 0, 8, 16, 24) give the 32 consecutive k of v_mfma_f32_32x32x64_f8f6f4.
+      const int krow = i16 >> 1;
+      const int chunk = (wn * 4 + grp) ^ (2 * krow);
+      r.b_base0 = (uint32_t)(kAStage256 + (32 * half + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
+    } else {
+      const int chunk = (wn * 8 + grp * 2 + (cq >> 1)) ^ (4 * t);
+      r.b_base0 = (uint32_t)(kAStage256 + (8 * half + t) * kBPitch + chunk * 16 + (cq & 1) * 8);
+    }
     return r;
+  }
+
+  typedef int i32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) i32x2 LdsPair;
+
+  // fp8 operands of k-block kk (64 k): A rows of slab b, B columns of block b.
+  TCCL_D Vec load_a8(const char* stage, const Reader& r, int kk, int b) const {
+    const int half = lane >> 5;
+    const char* p = stage + r.a_base + b * 32 * kARow256 + ((((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz) << 4);
+    const u32x4 lo = *(const u32x4*)p;
+    const u32x4 hi = *(const u32x4*)((uintptr_t)p ^ 16u);
+    typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+    const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(Vec, both);
+  }
+  TCCL_D Vec load_b8(const char* stage, const Reader& r, int kk, int b) const {
+    const char* p = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 32u)) + 64 * kk * kBPitch;
+    i32x2 q[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) q[t] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsPair*)(p + 8 * t * kBPitch));
+    i32x8 v;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[2 * t] = q[t][0];
+      v[2 * t + 1] = q[t][1];
+    }
+    return __builtin_bit_cast(Vec, v);
   }
 
   TCCL_D void load_frags(const char* stage, const Reader& r, int kk, Vec (&fa)[4], Vec (&fb)[2]) const {
@@ -224,9 +286,9 @@ struct Gemm256 {
     for (int b = 0; b < 4; ++b) fa[b] = *(const Vec*)(pa + b * 32 * kARow256);
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch256;
+      const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)pb);
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch256));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch));
       const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       fb[b] = __builtin_bit_cast(Vec, both);
     }
@@ -453,16 +515,36 @@ struct Gemm256 {
   TCCL_D void k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                      PullState& pull, char* pull_load, const char* pull_store) const {
     pull_step(pull, pa, pull_load, pull_store);
+    if constexpr (kFp8) {
+      // An fp8 operand is 8 registers: the A slabs are fetched one at a time so that the
+      // fragments in flight stay within what the 16-bit path holds.
 #pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      Vec fa[4], fb[2];
-      load_frags(cur, rd, kk, fa, fb);
-      issue_piece(nxt, src, kt_load, kk);
+      for (int kk = 0; kk < 2; ++kk) {
+        Vec fb[2];
+        fb[0] = load_b8(cur, rd, kk, 0);
+        fb[1] = load_b8(cur, rd, kk, 1);
+        issue_piece(nxt, src, kt_load, 2 * kk);
+        issue_piece(nxt, src, kt_load, 2 * kk + 1);
 #pragma unroll
-      for (int bi = 0; bi < 4; ++bi)
+        for (int bi = 0; bi < 4; ++bi) {
+          const Vec fa = load_a8(cur, rd, kk, bi);
+          acc[bi][0] = Mfma<InT>::run(fb[0], fa, acc[bi][0]);
+          acc[bi][1] = Mfma<InT>::run(fb[1], fa, acc[bi][1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = Mfma<InT>::run(fb[bj], fa[bi], acc[bi][bj]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int kk = 0; kk < 4; ++kk) {
+        Vec fa[4], fb[2];
+        load_frags(cur, rd, kk, fa, fb);
+        issue_piece(nxt, src, kt_load, kk);
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = Mfma<InT>::run(fb[bj], fa[bi], acc[bi][bj]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 
@@ -549,7 +631,7 @@ struct Gemm256 {
     // K steps are taken in pairs so that each call names its two stages statically and the
     // accumulators flow through one straight loop body.  An odd step count is rounded up: the
     // extra step (like the final look-ahead load) lies wholly past K and reads zeros.
-    const int ksteps = ((g.K + kBK - 1) / kBK + 1) & ~1;
+    const int ksteps = ((g.K + kStepK - 1) / kStepK + 1) & ~1;
     __syncthreads();  // the previous tile's epilogue has left LDS
 #pragma unroll
     for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);

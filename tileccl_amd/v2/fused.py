@@ -176,7 +176,9 @@ class FusedGemmAllGather(_FusedBase):
     def peer_out(self, peer: int) -> torch.Tensor:
         return self.heap.peer_view(self.out, peer)
 
-    def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0) -> torch.Tensor:
+    def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0,
+                 scale_a: float = 1.0, scale_b: float = 1.0) -> torch.Tensor:
+        alpha = float(alpha) * float(scale_a) * float(scale_b)  # per-tensor dequantisation scales of fp8 inputs
         gemm = _launch.gemm_desc(
             A, B, self.local_block, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
             alpha=alpha, num_wgs=self.num_gemm_wgs, macro_tile=self.macro_tile,
@@ -220,7 +222,9 @@ class FusedGemmReduceScatter(_FusedBase):
     def peer_out(self, peer: int) -> torch.Tensor:
         return self.heap.peer_view(self.out, peer)
 
-    def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0) -> torch.Tensor:
+    def __call__(self, A: torch.Tensor, B: torch.Tensor, variant: str = "s2", alpha: float = 1.0,
+                 scale_a: float = 1.0, scale_b: float = 1.0) -> torch.Tensor:
+        alpha = float(alpha) * float(scale_a) * float(scale_b)  # per-tensor dequantisation scales of fp8 inputs
         gemm = _launch.gemm_desc(
             A, B, self.partial, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
             alpha=alpha, num_wgs=self.num_gemm_wgs, macro_tile=self.macro_tile,
