@@ -101,9 +101,8 @@ __global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl:
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
   tccl::SignalArgs s;
   s.mode = tccl::kSignalNone;
-  tccl::PullArgs no_pull;
-  no_pull.peers = 0;
-  tccl::Gemm256<InT, OutT>(g, no_pull, -1, stage0, stage1, nullptr, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
+  tccl::PullArgs no_pull = {};  // mode 0: no background transfer
+  tccl::Gemm256<InT, OutT>(g, no_pull, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
 #endif
 }
 
@@ -129,10 +128,9 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
-  __shared__ __attribute__((aligned(16))) char pull0[tccl::kPullSlotBytes];
-  __shared__ __attribute__((aligned(16))) char pull1[tccl::kPullSlotBytes];
+  __shared__ __attribute__((aligned(16))) char landing[tccl::kBgBytes];
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
-  tccl::Gemm256<InT, OutT>(f.g, f.pull, (int)offsetof(Fused256Args, push), stage0, stage1, pull0, pull1)
+  tccl::Gemm256<InT, OutT>(f.g, f.pull, (int)offsetof(Fused256Args, push), stage0, stage1, landing)
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();
   const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));
@@ -388,24 +386,17 @@ int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 
-// The pull half of a TileGroup all-gather, as the large-tile K loop performs it in the
-// background.  Returns false when there is nothing of the kind to do.
-bool build_pull(const tccl::CommArgs& c, tccl::PullArgs* p) {
+// What the large-tile K loop can carry out in the background for a TileGroup launch: the
+// pull half of an all-gather, or a two-rank reduce-scatter.  Returns false when there is
+// nothing of the kind to do (the communication role after the last tile then does it).
+bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   memset(p, 0, sizeof *p);
-  if (c.op != tccl::kOpAllGather || c.granularity != tccl::kPerGroup || !(c.directions & tccl::kDirPull) || c.world <= 1) return false;
+  if (c.granularity != tccl::kPerGroup || c.world <= 1) return false;
   if (!c.row_ends || !c.tile_counts || !c.counter) return false;
   const int64_t row_bytes = (int64_t)c.N * c.esize;
-  const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
-  if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
-  p->peers = c.world - 1;
   p->rank = c.rank;
+  p->world = c.world;
   p->heap_bases = c.heap_bases;
-  p->block0_off = (int64_t)(uintptr_t)c.out - c.heap_bases[c.rank];
-  p->block_bytes = block_bytes;
-  p->pitch = (uint32_t)c.ld_out_bytes;
-  p->upr = (uint32_t)(row_bytes / 16);
-  p->units = (uint32_t)c.M * p->upr;
-  p->pieces = (int)((p->units + 63) / 64);
   p->counter = c.counter;
   p->row_ends = c.row_ends;
   p->tile_counts = c.tile_counts;
@@ -415,6 +406,41 @@ bool build_pull(const tccl::CommArgs& c, tccl::PullArgs* p) {
   p->trace_done_clock = c.trace_done_clock;
   p->fault = c.fault;
   p->spin_ticks = c.spin_ticks;
+  if (c.op == tccl::kOpAllGather) {
+    if (!(c.directions & tccl::kDirPull)) return false;
+    const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
+    if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
+    p->mode = tccl::kBgGather;
+    p->slots = c.world - 1;
+    p->src0 = c.out;
+    p->block_bytes = block_bytes;
+    p->block_rows = c.M;
+    p->pitch = (uint32_t)c.ld_out_bytes;
+  } else if (c.op == tccl::kOpReduceScatter) {
+    // two ranks only: the landing slots hold one addend per rank
+    if (c.world != 2 || c.M % 2) return false;
+    const int shard = c.M / 2;
+    const int64_t block_bytes = (int64_t)shard * c.ldc_bytes;
+    if (row_bytes % 16 || c.ldc_bytes % 16 || c.ld_rs_out_bytes % 8 || block_bytes >= (int64_t)1 << 32 ||
+        (int64_t)shard * c.ld_rs_out_bytes >= (int64_t)1 << 32)
+      return false;
+    if (c.out_dtype != tccl::kF16 && c.out_dtype != tccl::kBF16) return false;
+    p->mode = tccl::kBgReduce;
+    p->emulate_peer = c.emulate_peer;
+    p->slots = c.emulate_peer ? 2 : 1;
+    p->src0 = c.C;
+    p->block_bytes = block_bytes;
+    p->block_rows = shard;
+    p->pitch = (uint32_t)c.ldc_bytes;
+    p->dst0 = c.rs_out;
+    p->dst_pitch = (uint32_t)c.ld_rs_out_bytes;
+    p->out_bf16 = c.out_dtype == tccl::kBF16;
+  } else {
+    return false;
+  }
+  p->upr = (uint32_t)(row_bytes / 16);
+  p->units = (uint32_t)p->block_rows * p->upr;
+  p->pieces = (int)((p->units + 63) / 64);
   return true;
 }
 
@@ -424,9 +450,9 @@ bool build_push(const tccl::CommArgs& c, const tccl::GemmArgs& g, tccl::PushArgs
   memset(p, 0, sizeof *p);
   if (!(c.directions & tccl::kDirPush) || c.world <= 1) return false;
   if (c.op != tccl::kOpAllScatter && c.op != tccl::kOpAllGather) return false;
-  const int64_t mine = c.heap_bases[c.rank];
-  for (int q = 0; q < c.world; ++q)
-    if (q != c.rank) p->base[p->n++] = (char*)g.C + (c.heap_bases[q] - mine);
+  p->world = c.world;
+  p->rank = c.rank;
+  p->heap_bases = c.heap_bases;  // device memory: only the kernel reads it
   if (c.op == tccl::kOpAllScatter) {
     p->col_lo = c.src_col_off;
     p->col_hi = c.src_col_off + c.cols;
@@ -486,7 +512,12 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     // Pushes leave from the epilogue; what remains for the communication role are the
     // pulls (and, for a reduce-scatter, the reductions).
     if (build_push(c, g, &f.push)) c.directions &= ~tccl::kDirPush;
-    if (build_pull(c, &f.pull)) c.directions &= ~tccl::kDirPull;
+    if (build_background(c, &f.pull)) {
+      if (f.pull.mode == tccl::kBgReduce)
+        c.op = tccl::kOpNone;
+      else
+        c.directions &= ~tccl::kDirPull;
+    }
     if (c.op != tccl::kOpReduceScatter && !(c.directions & (tccl::kDirPush | tccl::kDirPull))) c.op = tccl::kOpNone;
     f.comm = c;
     return launch_fused256(d->in_dtype, d->out_dtype, f, wgs, stream);

@@ -69,36 +69,50 @@ struct Macro {
 // already sits in, instead of being written, signalled, re-read and copied by a second party
 // (reference: the per-tile scatter of patterns/_helpers.py:86-199, tile_allgather of
 // primitives/collectives.py:613-663).
-constexpr int kMaxPush = 7;
 struct PushArgs {
-  int n;               // number of targets; 0: the epilogue writes C only
+  int world;           // ranks; every rank but `rank` is a target.  0: the epilogue writes C only
+  int rank;
   int col_lo, col_hi;  // columns of C that travel
   int col_shift;       // target column = C column + col_shift
   int64_t ld;          // target pitch in elements
-  char* base[kMaxPush];  // address of C's (row 0, column 0) inside each target
+  const int64_t* heap_bases;  // C's address inside target q is C + heap_bases[q] - heap_bases[rank]
 };
 
-// The pull half of an all-gather, carried out in the shadow of the K loop (TileGroup variant).
-// A peer's block is cut into 1 KiB pieces (64 lanes x 16 bytes); wavefront w of the launch
-// owns pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid
-// sweeps a contiguous stretch of the block.  Each K step a wavefront stores the piece it
-// fetched during the previous step and fetches the next one straight into LDS; a piece is
-// fetched only once the TileGroups covering its rows are complete on the peer
-// (counter[g] >= epoch * tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66),
-// which is found out by a counter fetch that is itself left in flight for one K step.  What the
-// K loops did not get to is finished after the last tile, with bounded waits.
-// Groups must cover the block's rows in ascending order (build_tile_group_plan emits them so:
-// tileccl_v2/tile_group.py:244-301).
+// Background transfer: the part of the collective that reads finished TileGroups of the
+// peers, carried out in the shadow of the K loop (TileGroup variant).
+//   gather (all-gather pull):  out[block of peer] <- the peer's copy of that block
+//   reduce (reduce-scatter):   out_owner[row] = cast(partial_owner[row] + partial_other[row]), two ranks
+// A block (a peer's row block / an owner's shard of the partial) is cut into pieces of 64
+// units of 16 bytes; wavefront w of the launch owns pieces w, w + W, w + 2W, ... (W =
+// wavefronts in the grid), so at any moment the grid sweeps a contiguous stretch.  Each K
+// step a wavefront finishes the piece it fetched during the previous step (store it; or add
+// the two fetched addends in fp32, round once and store) and fetches the next one straight
+// into LDS.  A piece is fetched only once the TileGroups covering its rows are complete on
+// every rank it reads from (counter[g] >= epoch * tile_counts[g], the readiness rule of
+// tileccl_v2/signal.py:43-66); that is found out by counter fetches which are themselves
+// left in flight for one K step.  What the K loops did not get to is finished after the
+// last tile, with bounded waits.  Groups must cover the rows in ascending order and not
+// straddle a block border (build_tile_group_plan with row_split_boundaries emits them so:
+// tileccl_v2/tile_group.py:156-211, 244-301).
+enum BackgroundMode { kBgNone = 0, kBgGather = 1, kBgReduce = 2 };
 struct PullArgs {
-  int peers;                   // peers pulled from; 0 turns the background pull off
-  int rank;
+  int mode;
+  int slots;                   // blocks to process: gather: peers; reduce: owners handled here
+  int rank, world;
+  int emulate_peer;            // reduce: slot s is owner s (else the only slot is this rank's shard)
   const int64_t* heap_bases;
-  int64_t block0_off;          // slice offset of rank 0's block
-  int64_t block_bytes;         // distance between consecutive ranks' blocks (rows * pitch)
-  uint32_t pitch;              // bytes per row
-  uint32_t upr;                // 16-byte units per row
+  const char* src0;            // block 0 of the source in this rank's slice (gathered output / partial)
+  int64_t block_bytes;         // distance between consecutive blocks of the source (rows * pitch)
+  int block_rows;              // rows per block
+  uint32_t pitch;              // source bytes per row
+  uint32_t upr;                // 16-byte units per source row
   uint32_t units;              // units per block (rows * upr)
   int pieces;                  // pieces per block: ceil(units / 64)
+  // reduce only: the owner's output shard
+  const char* dst0;            // the output shard in this rank's slice
+  uint32_t dst_pitch;          // bytes per output row
+  int out_bf16;                // output element: 0 fp16, 1 bf16
+  // synchronisation
   const int32_t* counter;      // this rank's TileGroup counters; a peer's sit at the same slice offset
   const int32_t* row_ends;
   const int32_t* tile_counts;
@@ -108,8 +122,8 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
 };
-constexpr int kPullPieceBytes = 8 * 1024;                   // one 1 KiB landing slot per wavefront
-constexpr int kPullSlotBytes = kPullPieceBytes + 8 * 256;   // plus 256 B per wavefront for a fetched counter
+constexpr int kBgPieceBytes = 8 * 2048;                 // per wavefront two 1 KiB landing slots (gather uses one)
+constexpr int kBgBytes = kBgPieceBytes + 8 * 512;       // plus two fetched counter words (64 lanes x 4 B each)
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
   const int per_band = m.rows_per_band * m.cols;
@@ -160,13 +174,12 @@ struct Gemm256 {
   // are tracked per LDS variable, so a read of one stage need not wait for a load into the other.
   char* lds;   // stage 0 (also the epilogue's staging area)
   char* lds1;  // stage 1
-  char* bg0;   // landing slots of the background pull, one array per K-step parity
-  char* bg1;
+  char* bg;    // landing slots of the background transfer
   const int tid, lane, wave, wm, wn;
 
   TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, char* stage0, char* stage1,
-                 char* pull0, char* pull1)
-      : g(args), pa(pull_args), push_offset(push_args_offset), lds(stage0), lds1(stage1), bg0(pull0), bg1(pull1), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+                 char* landing)
+      : g(args), pa(pull_args), push_offset(push_args_offset), lds(stage0), lds1(stage1), bg(landing), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
         wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
@@ -294,19 +307,23 @@ struct Gemm256 {
     }
   }
 
-  // ---- background pull ---------------------------------------------------------------------------
+  // ---- background transfer -----------------------------------------------------------------------
   struct PullState {
-    int next_slot, next_lp;  // next piece of this wavefront: peer slot, piece inside the block
+    int next_slot, next_lp;  // next piece of this wavefront: block slot, piece inside the block
     int stride;              // wavefronts in the grid
-    int slot;                // peer slot that the bases and the readiness cache describe (-1: none)
-    int gidx;                // first TileGroup of that peer not yet known complete
-    uint32_t ready_units;    // units [0, ready_units) of that peer's block may be fetched
-    int64_t src_base, dst_base;
-    int64_t counter_base;    // address of that peer's counter words
-    int probe_group;         // group whose counter was fetched (into the landing slot) during the previous step; -1: none
+    int slot;                // slot that the bases and the readiness cache describe (-1: none)
+    int gidx;                // first TileGroup of that block not yet known complete
+    int row0;                // first row of that block in the plan's row numbering
+    uint32_t ready_units;    // units [0, ready_units) of that block may be fetched
+    int64_t src_base, src2_base, dst_base;  // addresses of the block in the slices involved
+    int64_t counter_base, counter2_base;    // the counter words of the ranks read from
+    int probe_group;         // group whose counters were fetched during the previous step (-1: none)
+    int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
+    uint32_t group_units;    // ready_units once group gidx is complete
+    int backoff;             // K steps to let pass before the counters are fetched again
     int pending_lp;          // piece fetched into LDS during the previous step (-1: none)
-    const char* pending_lds; // where it landed
-    int lds_off;             // this wavefront's landing slot inside a slot array
+    int lds_off;             // this wavefront's landing slots inside the landing array
+    int probe_off;           // and its counter landing words
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -318,60 +335,68 @@ struct Gemm256 {
   static TCCL_D T table(const T* p, int i) {
     return ((const __attribute__((address_space(4))) T*)p)[i];
   }
-  static TCCL_D int64_t uniform64(int64_t v) {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
-    return (int64_t)(((uint64_t)hi << 32) | lo);
-  }
+
+  TCCL_D bool bg_reduce() const { return pa.mode == kBgReduce; }
 
   TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
     PullState st;
     const int w = uniform(wave);
-    st.lds_off = w * 1024;
+    st.lds_off = w * 2048;
+    st.probe_off = kBgPieceBytes + w * 512;
     st.stride = num_wgs * (kThreads256 / 64);
     st.next_slot = 0;
     st.next_lp = wg * (kThreads256 / 64) + w;
     st.slot = -1;
     st.gidx = 0;
+    st.row0 = 0;
     st.ready_units = 0;
-    st.src_base = st.dst_base = st.counter_base = 0;
+    st.src_base = st.src2_base = st.dst_base = st.counter_base = st.counter2_base = 0;
     st.probe_group = -1;
+    st.need = 0;
+    st.group_units = 0;
+    st.backoff = 0;
     st.pending_lp = -1;
-    st.pending_lds = nullptr;
-    pull_normalise(st, a);
+    if (a.mode != kBgNone) pull_normalise(st, a);
     return st;
   }
 
-  // Fetch the first counter before the first tile's prologue, so that the first K step can
-  // already fetch a piece.  `landing` is the slot array that K step 0 reads.
+  // Fetch the first counters before the first tile's prologue, so that the first K step can
+  // already fetch a piece.
   TCCL_D void pull_prime(PullState& st, const PullArgs& a, char* landing) const {
-    if (a.peers == 0 || st.next_slot >= a.peers) return;
+    if (a.mode == kBgNone || st.next_slot >= a.slots) return;
     pull_select(st, a, st.next_slot);
     pull_probe(st, a, landing);
   }
 
+  // Every lane fetches the same word; it is read back from LDS one K step later.
   TCCL_D void pull_probe(PullState& st, const PullArgs& a, char* landing) const {
     if (st.gidx >= a.n_groups) return;
-    // every lane fetches the same word
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter_base), (LdsVoid*)(landing + kPullPieceBytes + (st.lds_off >> 2)), 4,
-                                             (uint32_t)st.gidx * 4u, 0, 0, kCoherent);
+    if (st.backoff > 0) {
+      --st.backoff;
+      return;
+    }
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter_base), (LdsVoid*)(landing + st.probe_off), 4, (uint32_t)st.gidx * 4u, 0, 0,
+                                             kCoherent);
+    if (a.mode == kBgReduce)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter2_base), (LdsVoid*)(landing + st.probe_off + 256), 4,
+                                               (uint32_t)st.gidx * 4u, 0, 0, kCoherent);
     st.probe_group = st.gidx;
   }
 
   TCCL_D void pull_normalise(PullState& st, const PullArgs& a) const {
-    while (st.next_lp >= a.pieces && st.next_slot < a.peers) {
+    while (st.next_lp >= a.pieces && st.next_slot < a.slots) {
       st.next_lp -= a.pieces;
       ++st.next_slot;
     }
   }
 
-  TCCL_D uint32_t pull_offset(const PullArgs& a, int lp, bool& valid) const {
+  // Row and 16-byte unit inside the row of this lane's unit of piece lp (row 0, unit 0 for idle lanes).
+  TCCL_D void pull_unit(const PullArgs& a, int lp, bool& valid, uint32_t& row, uint32_t& col) const {
     const uint32_t u = (uint32_t)lp * 64u + (uint32_t)lane;
     valid = u < a.units;
     const uint32_t uu = valid ? u : 0u;  // idle lanes touch the block's first unit and store nothing
-    if (a.pitch == a.upr * 16u) return uu * 16u;
-    const uint32_t row = uu / a.upr;
-    return row * a.pitch + (uu - row * a.upr) * 16u;
+    row = uu / a.upr;
+    col = uu - row * a.upr;
   }
 
   TCCL_D uint32_t pull_last_unit(const PullArgs& a, int lp) const {
@@ -381,107 +406,220 @@ struct Gemm256 {
 
   TCCL_D void pull_select(PullState& st, const PullArgs& a, int slot) const {
     if (slot == st.slot) return;
-    const int peer = slot < a.rank ? slot : slot + 1;
     st.slot = slot;
-    st.gidx = 0;
     st.ready_units = 0;
     st.probe_group = -1;
-    const int64_t rel = a.block0_off + (int64_t)peer * a.block_bytes;
-    const int64_t mine = table(a.heap_bases, a.rank), theirs = table(a.heap_bases, peer);
-    st.src_base = theirs + rel;
-    st.dst_base = mine + rel;
-    st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
+    st.backoff = 0;
+    const int64_t mine = table(a.heap_bases, a.rank);
+    if (a.mode == kBgGather) {
+      const int peer = slot < a.rank ? slot : slot + 1;
+      const int64_t theirs = table(a.heap_bases, peer);
+      const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)peer * a.block_bytes;
+      st.src_base = theirs + rel;
+      st.src2_base = 0;
+      st.dst_base = mine + rel;
+      st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
+      st.counter2_base = 0;
+      st.row0 = 0;  // the plan numbers the rows of one block
+      st.gidx = 0;
+      pull_group_facts(st, a);
+      return;
+    }
+    // reduce, two ranks: the owner's addend first, then the other rank's
+    const int owner = a.emulate_peer ? slot : a.rank;
+    const int other = 1 - owner;
+    const int64_t base_owner = table(a.heap_bases, owner), base_other = table(a.heap_bases, other);
+    const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)owner * a.block_bytes;
+    st.src_base = base_owner + rel;
+    st.src2_base = base_other + rel;
+    st.dst_base = base_owner + ((int64_t)(uintptr_t)a.dst0 - mine);
+    st.counter_base = (int64_t)(uintptr_t)a.counter;                  // this rank's own tiles
+    st.counter2_base = (int64_t)(uintptr_t)a.counter + (table(a.heap_bases, 1 - a.rank) - mine);
+    st.row0 = owner * a.block_rows;
+    int g = 0;
+    while (g < a.n_groups && table(a.row_ends, g) <= st.row0) ++g;  // the shard's first group
+    st.gidx = uniform(g);  // a loop's exit value does not count as uniform by itself
+    pull_group_facts(st, a);
   }
 
-  TCCL_D void pull_store_pending(PullState& st, const PullArgs& a, const char* slot_lds) const {
+  static TCCL_D void unpack(u32x4 v, float (&f)[8], int& n) {
+    if constexpr (sizeof(OutT) == 4) {
+      const f32x4v x = __builtin_bit_cast(f32x4v, v);
+      n = 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f[e] = x[e];
+        f[4 + e] = 0.f;
+      }
+    } else if constexpr (__is_same(OutT, __bf16)) {
+      const bf16x8v x = __builtin_bit_cast(bf16x8v, v);
+      n = 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)x[e];
+    } else {
+      const f16x8v x = __builtin_bit_cast(f16x8v, v);
+      n = 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)x[e];
+    }
+  }
+
+  // out = cast(first + second): fp32 sum, one rounding (tile_reduce_scatter, primitives/collectives.py:766-781).
+  TCCL_D void reduce_store(const PullArgs& a, const PullState& st, u32x4 first, u32x4 second, uint32_t row, uint32_t col, bool valid) const {
+    float x[8], y[8];
+    int n;
+    unpack(first, x, n);
+    unpack(second, y, n);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] += y[e];
+    const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
+    constexpr int kElems = 16 / sizeof(OutT);
+    const uint32_t off = row * a.dst_pitch + col * (kElems * 2);
+    if constexpr (kElems == 4) {
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      u32x2 w;
+      if (a.out_bf16) {
+        const __bf16 h[4] = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+        __builtin_memcpy(&w, h, 8);
+      } else {
+        const _Float16 h[4] = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+        __builtin_memcpy(&w, h, 8);
+      }
+      if (valid) __builtin_amdgcn_raw_buffer_store_b64(w, dst, off, 0, kStreaming);
+    } else {
+      const u32x4 w = a.out_bf16 ? pack8<__bf16>(x) : pack8<_Float16>(x);
+      if (valid) st16<kStreaming>(dst, off, w);
+    }
+  }
+
+  // Finish the piece that is sitting in the landing slots.
+  TCCL_D void pull_retire(PullState& st, const PullArgs& a, const char* landing) const {
     bool valid;
-    const uint32_t off = pull_offset(a, st.pending_lp, valid);
-    const u32x4 v = *(const u32x4*)(slot_lds + lane * 16);
-    if (valid) st16<kStreaming>(window(st.dst_base), off, v);
+    uint32_t row, col;
+    pull_unit(a, st.pending_lp, valid, row, col);
+    const u32x4 v = *(const u32x4*)(landing + st.lds_off + lane * 16);
+    if (a.mode == kBgGather) {
+      if (valid) st16<kStreaming>(window(st.dst_base), row * a.pitch + col * 16u, v);
+    } else {
+      const u32x4 v2 = *(const u32x4*)(landing + st.lds_off + 1024 + lane * 16);
+      reduce_store(a, st, v, v2, row, col, valid);
+    }
     st.pending_lp = -1;
   }
 
-  TCCL_D void pull_group_done(PullState& st, const PullArgs& a, int g) const {
-    st.ready_units = (uint32_t)table(a.row_ends, g) * a.upr;
-    st.gidx = g + 1;
+  // The two facts about group gidx that the per-step code needs, fetched when gidx changes.
+  TCCL_D void pull_group_facts(PullState& st, const PullArgs& a) const {
+    if (st.gidx >= a.n_groups) return;
+    st.need = a.epoch * table(a.tile_counts, st.gidx);
+    st.group_units = (uint32_t)(table(a.row_ends, st.gidx) - st.row0) * a.upr;
+  }
+  TCCL_D void pull_group_done(PullState& st, const PullArgs& a) const {
+    st.ready_units = st.group_units;
+    ++st.gidx;
+    pull_group_facts(st, a);
   }
 
-  // The per-K-step slice of the pull; all control flow here is wavefront-uniform.
-  TCCL_D void pull_step(PullState& st, const PullArgs& a, char* load_lds, const char* store_lds) const {
-    if (a.peers == 0) return;
-    if (st.pending_lp >= 0) pull_store_pending(st, a, store_lds + st.lds_off);
+  // The per-K-step slice of the transfer; all control flow here is wavefront-uniform.  One
+  // landing array serves every step: a slot is read back (and the read waited for) before
+  // the next fetch into it is issued, and the fetch has landed by the step's closing wait.
+  TCCL_D void pull_step(PullState& st, const PullArgs& a, char* landing) const {
+    if (a.mode == kBgNone) return;
+    if (st.pending_lp >= 0) pull_retire(st, a, landing);
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
       st.probe_group = -1;
-      const int32_t seen = uniform(*(const int32_t*)(store_lds + kPullPieceBytes + (st.lds_off >> 2)));
-      if (seen >= a.epoch * table(a.tile_counts, g)) pull_group_done(st, a, g);
+      int32_t seen = uniform(*(const int32_t*)(landing + st.probe_off));
+      if (a.mode == kBgReduce) {
+        const int32_t seen2 = uniform(*(const int32_t*)(landing + st.probe_off + 256));
+        seen = seen2 < seen ? seen2 : seen;
+      }
+      if (g == st.gidx) {
+        if (seen >= st.need)
+          pull_group_done(st, a);
+        else
+          st.backoff = 3;  // not there yet: fetching the counters every step only costs issue slots
+      }
     }
-    if (st.next_slot >= a.peers) return;
+    if (st.next_slot >= a.slots) return;
     if (st.next_slot != st.slot) {
       pull_select(st, a, st.next_slot);
-      pull_probe(st, a, load_lds);
+      pull_probe(st, a, landing);
       return;
     }
     if (pull_last_unit(a, st.next_lp) < st.ready_units) {
       bool valid;
-      const uint32_t off = pull_offset(a, st.next_lp, valid);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(load_lds + st.lds_off), 16, off, 0, 0, kCoherent);
+      uint32_t row, col;
+      pull_unit(a, st.next_lp, valid, row, col);
+      const uint32_t off = row * a.pitch + col * 16u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(landing + st.lds_off), 16, off, 0, 0, kCoherent);
+      if (a.mode == kBgReduce)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src2_base), (LdsVoid*)(landing + st.lds_off + 1024), 16, off, 0, 0, kCoherent);
       st.pending_lp = st.next_lp;
-      st.pending_lds = load_lds + st.lds_off;
       st.next_lp += st.stride;
       pull_normalise(st, a);
     }
-    pull_probe(st, a, load_lds);  // look ahead: the next group's counter
+    pull_probe(st, a, landing);  // look ahead: the next group's counters
   }
 
-  // Wait (bounded) until units [0, last] of the selected peer's block may be fetched.
+  // Wait (bounded) until units [0, last] of the selected block may be fetched.
   TCCL_D bool pull_wait_ready(PullState& st, const PullArgs& a, uint32_t last, int64_t deadline) const {
     while (last >= st.ready_units) {
       if (st.gidx >= a.n_groups) return false;
-      const int32_t need = a.epoch * table(a.tile_counts, st.gidx);
+      const int32_t need = st.need;
       const __amdgpu_buffer_rsrc_t words = window(st.counter_base);
+      const __amdgpu_buffer_rsrc_t words2 = window(a.mode == kBgReduce ? st.counter2_base : st.counter_base);
       for (;;) {
         const int32_t seen = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(words, (uint32_t)st.gidx * 4u, 0, kCoherent);
-        if (uniform(seen) >= need) break;
+        const int32_t seen2 = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(words2, (uint32_t)st.gidx * 4u, 0, kCoherent);
+        if (uniform(seen) >= need && uniform(seen2) >= need) break;
         if (now_ticks() > deadline) return false;
         __builtin_amdgcn_s_sleep(8);
       }
-      pull_group_done(st, a, st.gidx);
+      pull_group_done(st, a);
     }
     return true;
   }
 
-  // After the last tile: store what is in flight, move the remaining pieces, report.
-  TCCL_D void pull_finish(PullState& st, const PullArgs& a, int num_wgs) const {
-    if (a.peers == 0) return;
+  // After the last tile: finish what is in flight, move the remaining pieces, report.
+  TCCL_D void pull_finish(PullState& st, const PullArgs& a, const char* landing, int num_wgs) const {
+    if (a.mode == kBgNone) return;
     wait_vmem();
-    if (st.pending_lp >= 0) pull_store_pending(st, a, st.pending_lds);
+    if (st.pending_lp >= 0) pull_retire(st, a, landing);
     st.probe_group = -1;
     const int64_t deadline = now_ticks() + a.spin_ticks;
     bool ok = true;
-    constexpr int kBatch = 4;
-    while (ok && st.next_slot < a.peers) {
+    constexpr int kBatch = 8;  // pieces in flight per wavefront: the CU has no other work left
+    while (ok && st.next_slot < a.slots) {
       pull_select(st, a, st.next_slot);
-      u32x4 v[kBatch];
-      uint32_t off[kBatch];
-      bool valid[kBatch];
+      u32x4 v[kBatch], v2[kBatch];
+      uint32_t row[kBatch], col[kBatch];
+      bool valid[kBatch], loaded[kBatch];
       int n = 0;
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
-        valid[k] = false;
+        valid[k] = loaded[k] = false;
         const int lp = st.next_lp + k * st.stride;
         if (ok && lp < a.pieces) {
           ok = pull_wait_ready(st, a, pull_last_unit(a, lp), deadline);
           if (ok) {
-            off[k] = pull_offset(a, lp, valid[k]);
-            v[k] = ld16<kCoherent>(window(st.src_base), off[k]);
+            pull_unit(a, lp, valid[k], row[k], col[k]);
+            const uint32_t off = row[k] * a.pitch + col[k] * 16u;
+            v[k] = ld16<kCoherent>(window(st.src_base), off);
+            if (a.mode == kBgReduce) v2[k] = ld16<kCoherent>(window(st.src2_base), off);
+            loaded[k] = true;
             n = k + 1;
           }
         }
       }
 #pragma unroll
-      for (int k = 0; k < kBatch; ++k)
-        if (valid[k]) st16<kStreaming>(window(st.dst_base), off[k], v[k]);
+      for (int k = 0; k < kBatch; ++k) {
+        if (!loaded[k]) continue;
+        if (a.mode == kBgGather) {
+          if (valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a.pitch + col[k] * 16u, v[k]);
+        } else {
+          reduce_store(a, st, v[k], v2[k], row[k], col[k], valid[k]);
+        }
+      }
       st.next_lp += n * st.stride;
       if (n < kBatch) {  // the block is finished (or a wait gave up)
         st.next_lp -= a.pieces;
@@ -513,8 +651,8 @@ struct Gemm256 {
   // spill reloads would drain the load queue every step.  The scheduling barrier keeps the
   // compiler from hoisting the next chunk's reads across the MFMAs.
   TCCL_D void k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
-                     PullState& pull, char* pull_load, const char* pull_store) const {
-    pull_step(pull, pa, pull_load, pull_store);
+                     PullState& pull) const {
+    pull_step(pull, pa, bg);
     if constexpr (kFp8) {
       // An fp8 operand is 8 registers: the A slabs are fetched one at a time so that the
       // fragments in flight stay within what the 16-bit path holds.
@@ -548,6 +686,7 @@ struct Gemm256 {
     }
   }
 
+  // Stores the tile and, when a push is asked for, sends it to the peers from the same LDS staging.
   template <int kPolicy>
   TCCL_D void epilogue(int row0, int col0, const f32x16 (&acc)[4][2]) const {
     constexpr int kEsz = sizeof(OutT);
@@ -558,10 +697,10 @@ struct Gemm256 {
     const int half = lane >> 5, l32 = lane & 31;
     OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
     const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
-    // Fields are read through the argument block itself: a local copy of base[] would be
-    // indexed dynamically and end up in scratch memory.
+    // Fields are read through the argument block itself: a local copy would sit in scalar
+    // registers all through the K loop.
     const auto* push = late_kernarg_ptr<PushArgs>(push_offset < 0 ? 0 : push_offset);
-    const int push_n = push_offset >= 0 ? push->n : 0;
+    const int push_world = push_offset >= 0 ? push->world : 0;
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
       __syncthreads();
@@ -601,10 +740,12 @@ struct Gemm256 {
         live[r] = row0 + lrow[r] < g.M && col0 + lcol[r] < g.N;
         if (live[r]) __builtin_amdgcn_raw_buffer_store_b128(v[r], rc, (uint32_t)((lrow[r] * g.ldc + lcol[r]) * kEsz), 0, kPolicy);
       }
-      for (int t = 0; t < push_n; ++t) {
+      for (int t = 0; t < push_world; ++t) {
+        if (t == push->rank) continue;
         const int64_t push_ld = push->ld;
         const int col_lo = push->col_lo, col_hi = push->col_hi;
-        char* base = push->base[t] + ((int64_t)row0 * push_ld + col0 + push->col_shift) * kEsz;
+        const int64_t delta = table(push->heap_bases, t) - table(push->heap_bases, push->rank);
+        char* base = (char*)g.C + delta + ((int64_t)row0 * push_ld + col0 + push->col_shift) * kEsz;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffffu, 0x00020000);
 #pragma unroll
         for (int r = 0; r < kRounds; ++r) {
@@ -617,7 +758,8 @@ struct Gemm256 {
   }
 
   template <int kPolicy>
-  TCCL_D void macro_tile(int row0, int col0, PullState& pull) const {
+  TCCL_D void macro_tile(const SignalArgs& s, int mm, int mn, PullState& pull) const {
+    const int row0 = mm * kMacro, col0 = mn * kMacro;
     f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -638,17 +780,21 @@ struct Gemm256 {
     wait_vmem();
     __syncthreads();
     for (int kt = 0; kt < ksteps; kt += 2) {
-      k_step(lds, lds1, src, rd, kt + 1, acc, pull, bg0, bg1);
+      k_step(lds, lds1, src, rd, kt + 1, acc, pull);
       wait_vmem();
       __syncthreads();
-      k_step(lds1, lds, src, rd, kt + 2, acc, pull, bg1, bg0);
+      k_step(lds1, lds, src, rd, kt + 2, acc, pull);
       wait_vmem();
       __syncthreads();
     }
     epilogue<kPolicy>(row0, col0, acc);
+    if constexpr (kPolicy != 0) {
+      wait_vmem();  // the tile's write-through stores have landed
+      __syncthreads();
+      if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+    }
   }
 
-  // Publish every plan tile the macro tile (mm, mn) covers.
   // Plan tiles of one row share a TileGroup, so the group counts are summed up here and
   // each group gets one add (concurrent adds to one word serialise).
   TCCL_D void publish(const SignalArgs& s, int mm, int mn) const {
@@ -677,21 +823,16 @@ struct Gemm256 {
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
     const int total = m.rows * m.cols;
     PullState pull = pull_begin(pa, wg, num_wgs);
-    pull_prime(pull, pa, bg1);
+    pull_prime(pull, pa, bg);
     for (int slot = wg; slot < total; slot += num_wgs) {
       const int id = tile_for_slot(slot, total, m.xcds, m.span);
       const TileCoord c = macro_coords(id, m);
-      const int row0 = c.m * kMacro, col0 = c.n * kMacro;
-      if (s.mode == kSignalNone && push_offset < 0) {
-        macro_tile<0>(row0, col0, pull);
-      } else {
-        macro_tile<kCoherent>(row0, col0, pull);
-        wait_vmem();
-        __syncthreads();
-        if (tid == 0 && s.mode != kSignalNone) publish(s, c.m, c.n);
-      }
+      if (s.mode == kSignalNone && push_offset < 0)
+        macro_tile<0>(s, c.m, c.n, pull);
+      else
+        macro_tile<kCoherent>(s, c.m, c.n, pull);
     }
-    pull_finish(pull, pa, num_wgs);
+    pull_finish(pull, pa, bg, num_wgs);
   }
 };
 #endif  // __HIP_DEVICE_COMPILE__
