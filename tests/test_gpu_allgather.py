@@ -181,6 +181,39 @@ def test_pull_with_padded_rows_and_short_k(lib):
             h.cleanup()
 
 
+@pytest.mark.parametrize("macro", MACRO)
+def test_device_trace_of_a_tilegroup_launch(lib, macro):
+    """A traced S2 launch leaves, per TileGroup, start <= ready <= done clocks; the recorder
+    turns them into one produce and one transfer span per group."""
+    from tileccl_amd.v2.runtime import TimelineRecorder
+
+    M, N, K = 1024, 512, 256
+    heaps, ops = make(2, M, N, macro_tile=macro, trace=True, tau_min_bytes=1, group_m=2)
+    try:
+        op = ops[0]
+        assert op.plan.n_groups == 4
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=K**-0.5))
+        fill_peer_blocks(ops, M, N, torch.float16)
+        op.mark_peers_ready()
+        op.signals.trace_start_clock.zero_()
+        op.signals.trace_ready_clock.zero_()
+        op.signals.trace_done_clock.zero_()
+        op(A, B, "s2")
+        op.check_faults()
+        t0 = int(op.signals.trace_start_clock.cpu()[0])
+        ready, done = op.signals.trace_ready_clock.cpu().tolist(), op.signals.trace_done_clock.cpu().tolist()
+        assert t0 > 0
+        for g in range(4):
+            assert t0 <= ready[g] <= done[g], (g, t0, ready, done)
+        rec = TimelineRecorder(benchmark="gemm_allgather", path_name=f"s2 macro {macro}")
+        made = rec.record_signal_state(op.signals, op.plan, rank=0)
+        assert len(made) == 8 and rec.to_payload()["lane_order"] == [f"group {g}" for g in range(4)]
+        assert all(e.end_ms < 50.0 for e in made)  # milliseconds: a sub-millisecond launch
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
 def test_single_rank_is_a_plain_gemm(lib):
     heaps, ops = make(1, 256, 256)
     try:

@@ -506,6 +506,9 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
       s.mode = tccl::kSignalGroup;
       s.counter = sync->counter;
       s.group_table = sync->group_table;
+      s.tile_counts = sync->tile_counts;
+      s.epoch = sync->epoch > 0 ? sync->epoch : 1;
+      s.trace_ready_clock = sync->trace_ready_clock;
       c.granularity = tccl::kPerGroup;
     }
     f.s = s;

@@ -61,6 +61,10 @@ struct SignalArgs {
   int32_t* locks;
   const int32_t* group_table;
   int32_t* counter;
+  // optional device trace: the producer that completes a group stamps its clock
+  const int32_t* tile_counts;
+  int epoch;
+  int64_t* trace_ready_clock;
 };
 
 template <typename T>

@@ -811,13 +811,18 @@ struct Gemm256 {
         }
         const int gi = s.group_table[tile_id];
         if (gi != group && count > 0) {
-          tile_signal_add<true>(s.counter, group, count);
+          add_to_group(s, group, count);
           count = 0;
         }
         group = gi;
         ++count;
       }
-    if (count > 0) tile_signal_add<true>(s.counter, group, count);
+    if (count > 0) add_to_group(s, group, count);
+  }
+
+  TCCL_D void add_to_group(const SignalArgs& s, int group, int count) const {
+    const int32_t prev = tile_signal_add<true>(s.counter, group, count);
+    if (s.trace_ready_clock && prev + count == s.epoch * s.tile_counts[group]) s.trace_ready_clock[group] = now_ticks();
   }
 
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
