@@ -1,0 +1,114 @@
+"""``tileccl.ops.gemm_allgather`` / ``gemm_reducescatter`` (column shards) on the HIP kernels,
+against the CPU oracle; world size 2 and 3 emulated as slices of one arena."""
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import assert_gemm_close, bits, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def contexts(world, heap_bytes=128 << 20):
+    import tileccl_amd as tileccl
+
+    return tileccl.init_local(world_size=world, heap_size=heap_bytes)
+
+
+def put(ctx, cpu):
+    t = ctx.zeros(*cpu.shape, dtype=cpu.dtype)
+    t.copy_(cpu)
+    return t
+
+
+@pytest.mark.parametrize("variant", ["s0", "s1", "s2"])
+@pytest.mark.parametrize("world,M,N,K", [(2, 512, 512, 256), (3, 300, 768, 72), (2, 4096, 4096, 512)])
+def test_gemm_allgather_column_shards(lib, variant, world, M, N, K):
+    import tileccl_amd as tileccl
+
+    ctxs = contexts(world, 256 << 20)
+    try:
+        Ns = N // world
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        As = [put(c, A_cpu) for c in ctxs]
+        Bs = [put(c, B_cpu[:, r * Ns:(r + 1) * Ns].contiguous()) for r, c in enumerate(ctxs)]
+        Cs = [c.zeros(M, N, dtype=torch.float16) for c in ctxs]
+        for r, c in enumerate(ctxs):
+            out = tileccl.ops.gemm_allgather(As[r], Bs[r], Cs[r], ctx=c, variant=variant)
+            assert out is Cs[r]
+        torch.cuda.synchronize()
+        # every rank holds the same full product, bit for bit
+        for r in range(1, world):
+            assert torch.equal(bits(Cs[0]), bits(Cs[r]))
+        assert_gemm_close(Cs[0], A_cpu.float() @ B_cpu.float(), tight=0.004)
+        # each column block is the bytes its owner's GEMM produced: compare with the oracle per block
+        for r in range(world):
+            want = oracle.gemm(A_cpu, B_cpu[:, r * Ns:(r + 1) * Ns], torch.float16)
+            assert (Cs[0][:, r * Ns:(r + 1) * Ns].cpu().float() - want.float()).abs().max().item() <= 0.004
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()
+
+
+@pytest.mark.parametrize("world,M,N,K", [(2, 512, 512, 256), (2, 200, 272, 72), (3, 256, 768, 128)])
+def test_gemm_reducescatter_column_shards(lib, world, M, N, K):
+    import tileccl_amd as tileccl
+
+    ctxs = contexts(world)
+    try:
+        Ns = N // world
+        A_cpu = [seeded((M, K), 10 + r) for r in range(world)]
+        B_cpu = seeded((K, N), 1, scale=K**-0.5)
+        As = [put(c, A_cpu[r]) for r, c in enumerate(ctxs)]
+        Bs = [put(c, B_cpu) for c in ctxs]
+        Cs = [c.zeros(M, Ns, dtype=torch.float16) for c in ctxs]
+        # Emulation: a rank's partial is resident once its op has run, so run the round twice;
+        # after the second round every rank has reduced over final partials.
+        for _ in range(2):
+            for r, c in enumerate(ctxs):
+                assert tileccl.ops.gemm_reducescatter(As[r], Bs[r], Cs[r], ctx=c) is Cs[r]
+        torch.cuda.synchronize()
+        full = sum(a.float() @ B_cpu.float() for a in A_cpu)
+        partials = [c.workspace("gemm_reducescatter.partial", world, M, Ns, dtype=torch.float32).cpu() for c in ctxs]
+        for r in range(world):
+            assert_gemm_close(Cs[r], full[:, r * Ns:(r + 1) * Ns], tight=0.006)
+            # bit-exact against the oracle's reduction of the partials the GPU produced
+            tall = [p.reshape(world * M, Ns) for p in partials]
+            want = oracle.reduce_rows(tall, r, torch.float16)
+            if world == 2:
+                assert torch.equal(bits(Cs[r]).cpu(), bits(want))
+            else:
+                assert (Cs[r].cpu().float() - want.float()).abs().max().item() <= 0.002
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()
+
+
+def test_contract_errors(lib):
+    import tileccl_amd as tileccl
+
+    ctxs = contexts(2, 16 << 20)
+    try:
+        c = ctxs[0]
+        A, B, Cf = c.zeros(128, 64, dtype=torch.float16), c.zeros(64, 128, dtype=torch.float16), c.zeros(128, 256, dtype=torch.float16)
+        with pytest.raises(ValueError, match=r"gemm_allgather expects 2-D tensors: got A.ndim=1"):
+            tileccl.ops.gemm_allgather(A[0], B, Cf, ctx=c)
+        with pytest.raises(ValueError, match="RHS shard columns must match the rank-local shard width: expected 128, got 64"):
+            tileccl.ops.gemm_allgather(A, B[:, :64].contiguous(), Cf, ctx=c)
+        with pytest.raises(ValueError, match=r"requires C.shape\[1\] to be divisible by world_size: 255 % 2 != 0"):
+            tileccl.ops.gemm_allgather(A, B, c.zeros(128, 255, dtype=torch.float16), ctx=c)
+        with pytest.raises(ValueError, match="share one dtype"):
+            tileccl.ops.gemm_allgather(A, B, c.zeros(128, 256, dtype=torch.bfloat16), ctx=c)
+        with pytest.raises(ValueError, match="C must reside in the attached symmetric heap"):
+            tileccl.ops.gemm_allgather(A, B, torch.zeros(128, 256, dtype=torch.float16, device="cuda"), ctx=c)
+        with pytest.raises(ValueError, match="unknown variant 's7'"):
+            tileccl.ops.gemm_allgather(A, B, Cf, ctx=c, variant="s7")
+        Bf = c.zeros(64, 256, dtype=torch.float16)
+        with pytest.raises(ValueError, match="output columns must match the rank-local shard width: expected 128, got 256"):
+            tileccl.ops.gemm_reducescatter(A, Bf, Cf, ctx=c)
+        with pytest.raises(ValueError, match=r"B.shape\[0\] must equal A.shape\[1\]: got 32 vs 64"):
+            tileccl.ops.gemm_reducescatter(A, Bf[:32], c.zeros(128, 128, dtype=torch.float16), ctx=c)
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()

@@ -26,6 +26,8 @@ from tileccl_amd.patterns import (
 from tileccl_amd.patterns.contracts import PatternExecutionSpec, resolve_pattern_execution
 
 __all__ = [
+    "gemm_allgather",
+    "gemm_reducescatter",
     "gemm_allscatter",
     "gemm_allscatter_sharded",
     "build_gemm_allscatter_plan",
@@ -33,6 +35,8 @@ __all__ = [
     "GemmAllScatterMixedLayoutPlan",
     "GemmAllScatterContract",
 ]
+
+from tileccl_amd.ops_collective import gemm_allgather, gemm_reducescatter  # noqa: E402  (re-exported)
 
 PatternLike = str | type[Pattern] | Pattern | None
 LayoutKind = Literal["full", "shard"]
