@@ -115,3 +115,30 @@ def test_v2_heap(lib):
     finally:
         for h in heaps:
             h.cleanup()
+
+
+def test_cost_model_calibration_on_the_device(lib):
+    """Transfers of growing size through the C ABI, fitted by CostModelCalibrator: the fitted
+    line must explain the large transfers and give a sane bandwidth for copies inside one HBM."""
+    from tileccl_amd.v2 import SymmetricHeap
+    from tileccl_amd.v2.calibrate import calibrate
+
+    heaps = SymmetricHeap.create_all(512 << 20, 2)
+    try:
+        cal = calibrate(heaps[0], gemm_shape=(2048, 2048, 512))
+        sizes = [p.nbytes for p in cal.points]
+        assert sizes == sorted(sizes) and sizes[0] == 8192 and sizes[-1] == 32 << 20
+        times = [p.measured_comm_us for p in cal.points]
+        assert all(t > 0 for t in times) and times[-1] > times[0]
+        prof = cal.profile
+        assert 200.0 < prof.bandwidth_gb_s < 8000.0  # push = read + write of the payload through one HBM
+        assert 0.5 < prof.min_comm_us < 50.0  # launch latency floor, microseconds
+        big = cal.points[-1]
+        predicted = max(prof.min_comm_us, prof.alpha_us + big.nbytes * prof.beta_us_per_byte)
+        assert abs(predicted - big.measured_comm_us) / big.measured_comm_us < 0.25
+        assert 50.0 < cal.gemm_tflops < 2500.0 and 0.0 < prof.gemm_efficiency <= 1.0
+        tiles = cal.target_group_tiles(4096, 4096, 1024)
+        assert tiles % (8 * 32) == 0 and 256 <= tiles <= 1024  # whole swizzle waves of the 4096 x 4096 plan
+    finally:
+        for h in heaps:
+            h.cleanup()
