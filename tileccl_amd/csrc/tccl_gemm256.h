@@ -292,11 +292,12 @@ struct Gemm256 {
     return __builtin_bit_cast(Vec, v);
   }
 
-  TCCL_D void load_frags(const char* stage, const Reader& r, int kk, Vec (&fa)[4], Vec (&fb)[2]) const {
+  // 16-bit operands of k-block kk (16 k): the A rows of slab bi; the B columns of both blocks.
+  TCCL_D Vec load_a16(const char* stage, const Reader& r, int kk, int bi) const {
     const int half = lane >> 5;
-    const char* pa = stage + r.a_base + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4);
-#pragma unroll
-    for (int b = 0; b < 4; ++b) fa[b] = *(const Vec*)(pa + b * 32 * kARow256);
+    return *(const Vec*)(stage + r.a_base + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4) + bi * 32 * kARow256);
+  }
+  TCCL_D void load_b16(const char* stage, const Reader& r, int kk, Vec (&fb)[2]) const {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch;
@@ -672,15 +673,28 @@ struct Gemm256 {
         __builtin_amdgcn_sched_barrier(0);
       }
     } else {
+      // Sixteen items (k-block kk, A slab bi) of two MFMAs each.  The operands of item i + 2
+      // are fetched before the MFMAs of item i are issued, so an LDS read has two items
+      // (~130 clocks of matrix work, more with the SIMD's other wave) to come back; measured
+      // with whole k-blocks fetched and consumed in turn, LDS latency and MFMA time simply
+      // added up.  A rotates through three registers sets, B through two; the scheduling
+      // barriers pin this order (left alone, the compiler hoists every read of the step and
+      // spills).
+      Vec ring[3], fbr[2][2];
+      load_b16(cur, rd, 0, fbr[0]);
+      ring[0] = load_a16(cur, rd, 0, 0);
+      ring[1] = load_a16(cur, rd, 0, 1);
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        Vec fa[4], fb[2];
-        load_frags(cur, rd, kk, fa, fb);
-        issue_piece(nxt, src, kt_load, kk);
-#pragma unroll
-        for (int bi = 0; bi < 4; ++bi)
-#pragma unroll
-          for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = Mfma<InT>::run(fb[bj], fa[bi], acc[bi][bj]);
+      for (int i = 0; i < 16; ++i) {
+        const int kk = i >> 2, bi = i & 3;
+        if (i + 2 < 16) {
+          const int j = i + 2;
+          if ((j & 3) == 0) load_b16(cur, rd, j >> 2, fbr[(j >> 2) & 1]);
+          ring[j % 3] = load_a16(cur, rd, j >> 2, j & 3);
+        }
+        if (bi == 0) issue_piece(nxt, src, kt_load, kk);
+        acc[bi][0] = Mfma<InT>::run(fbr[kk & 1][0], ring[i % 3], acc[bi][0]);
+        acc[bi][1] = Mfma<InT>::run(fbr[kk & 1][1], ring[i % 3], acc[bi][1]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
