@@ -53,9 +53,10 @@ def test_small_two_ranks_bit_exact(lib, variant, partial_dtype, out_dtype, macro
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-def test_without_peer_emulation_only_the_own_shard_is_written(lib, variant):
+@pytest.mark.parametrize("macro", [128, 256])
+def test_without_peer_emulation_only_the_own_shard_is_written(lib, variant, macro):
     M, N, K = 512, 256, 64
-    heaps, ops = make(2, M, N, emulate_peer=False)
+    heaps, ops = make(2, M, N, emulate_peer=False, macro_tile=macro)
     try:
         A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=1 / 8))
         peer = seeded((M, N), 2, torch.float32)
@@ -74,10 +75,13 @@ def test_without_peer_emulation_only_the_own_shard_is_written(lib, variant):
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-def test_three_ranks_sum_order_owner_first(lib, variant):
-    """With three addends the fp32 sum depends on order: owner first, then ascending ranks."""
-    M, N, K = 768, 264, 64
-    heaps, ops = make(3, M, N, tau_min_bytes=1, group_m=1)
+@pytest.mark.parametrize("macro,M", [(128, 768), (256, 768), (256, 384)])
+def test_three_ranks_sum_order_owner_first(lib, variant, macro, M):
+    """With three addends the fp32 sum depends on order: owner first, then ascending ranks.
+    M = 768 gives shards of whole 256-row tiles (the large-tile kernel reduces tile by tile);
+    M = 384 gives 128-row shards (it reduces after its last tile instead)."""
+    N, K = 264, 64
+    heaps, ops = make(3, M, N, tau_min_bytes=1, group_m=1, macro_tile=macro)
     try:
         A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=1 / 8))
         peers = {p: seeded((M, N), 10 + p, torch.float32) * 1000.0 for p in (1, 2)}  # large magnitudes: order matters
@@ -124,6 +128,26 @@ def test_baseline_config_3_properties(lib):
         rows = slice(4000, 4128)
         assert_gemm_close(op.partial[rows], A[rows].float().cpu() @ B.float().cpu(), tight=1e-3)
         assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
+@pytest.mark.parametrize("variant", ["s1", "s2"])
+def test_tile_by_tile_reduce_gives_up_when_the_peer_never_publishes(lib, variant):
+    """Large-tile kernel, own rows, a peer whose words stay at zero: the bounded wait expires,
+    the launch ends normally with the partial complete, and the host raises."""
+    M, N, K = 512, 256, 64
+    heaps, ops = make(2, M, N, emulate_peer=False, macro_tile=256, spin_limit_ns=200_000)
+    try:
+        A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=1 / 8))
+        ops[0](A, B, variant)
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            ops[0].check_faults()
+        assert_gemm_close(ops[0].partial, A.float().cpu() @ B.float().cpu(), tight=1e-3)
+        ops[0].mark_peers_ready()
+        ops[0](A, B, variant)
+        ops[0].check_faults()
     finally:
         for h in heaps:
             h.cleanup()

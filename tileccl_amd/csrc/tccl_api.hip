@@ -102,7 +102,7 @@ __global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl:
   tccl::SignalArgs s;
   s.mode = tccl::kSignalNone;
   tccl::PullArgs no_pull = {};  // mode 0: no background transfer
-  tccl::Gemm256<InT, OutT>(g, no_pull, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
+  tccl::Gemm256<InT, OutT>(g, no_pull, -1, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
 #endif
 }
 
@@ -120,17 +120,19 @@ struct Fused256Args {
   int64_t* trace_start;
   tccl::PullArgs pull;
   tccl::PushArgs push;
+  tccl::ReduceArgs reduce;
   tccl::CommArgs comm;
 };
 
-template <typename InT, typename OutT>
+template <typename InT, typename OutT, bool kWithReduce>
 __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char landing[tccl::kBgBytes];
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
-  tccl::Gemm256<InT, OutT>(f.g, f.pull, (int)offsetof(Fused256Args, push), stage0, stage1, landing)
+  tccl::Gemm256<InT, OutT, kWithReduce>(f.g, f.pull, (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
+                                        landing)
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();
   const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));
@@ -340,6 +342,7 @@ tccl::Macro build_macro(const tccl_gemm_desc* d, const tccl_device_info& dev, in
   int span = in_flight / (dev.xcds > 0 ? dev.xcds : 1);
   span = span / m.rows_per_band * m.rows_per_band;
   m.span = span > 0 ? span : 1;
+  m.row_shift = 0;
   return m;
 }
 
@@ -370,7 +373,12 @@ int launch_gemm256(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const t
 
 template <typename InT, typename OutT>
 int launch_fused256_t(const Fused256Args& f, int wgs, hipStream_t stream) {
-  hipLaunchKernelGGL((fused256_kernel<InT, OutT>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
+  // The tile-by-tile reduce-scatter is a separate instantiation: its code would otherwise
+  // raise the register pressure of every fused kernel.
+  if (f.reduce.active)
+    hipLaunchKernelGGL((fused256_kernel<InT, OutT, true>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
+  else
+    hipLaunchKernelGGL((fused256_kernel<InT, OutT, false>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
   TCCL_HIP(hipGetLastError());
   return 0;
 }
@@ -386,17 +394,28 @@ int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 
-// What the large-tile K loop can carry out in the background for a TileGroup launch: the
-// pull half of an all-gather, or a two-rank reduce-scatter.  Returns false when there is
-// nothing of the kind to do (the communication role after the last tile then does it).
+// The pull half of a TileGroup all-gather, as the large-tile K loop performs it in the
+// background.  Returns false when there is nothing of the kind to do (the communication role
+// after the last tile then does it).
 bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   memset(p, 0, sizeof *p);
-  if (c.granularity != tccl::kPerGroup || c.world <= 1) return false;
+  if (c.op != tccl::kOpAllGather || c.granularity != tccl::kPerGroup || !(c.directions & tccl::kDirPull) || c.world <= 1) return false;
   if (!c.row_ends || !c.tile_counts || !c.counter) return false;
   const int64_t row_bytes = (int64_t)c.N * c.esize;
+  const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
+  if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
+  p->mode = tccl::kBgGather;
+  p->slots = c.world - 1;
   p->rank = c.rank;
   p->world = c.world;
   p->heap_bases = c.heap_bases;
+  p->src0 = c.out;
+  p->block_bytes = block_bytes;
+  p->block_rows = c.M;
+  p->pitch = (uint32_t)c.ld_out_bytes;
+  p->upr = (uint32_t)(row_bytes / 16);
+  p->units = (uint32_t)p->block_rows * p->upr;
+  p->pieces = (int)((p->units + 63) / 64);
   p->counter = c.counter;
   p->row_ends = c.row_ends;
   p->tile_counts = c.tile_counts;
@@ -406,41 +425,33 @@ bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   p->trace_done_clock = c.trace_done_clock;
   p->fault = c.fault;
   p->spin_ticks = c.spin_ticks;
-  if (c.op == tccl::kOpAllGather) {
-    if (!(c.directions & tccl::kDirPull)) return false;
-    const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
-    if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
-    p->mode = tccl::kBgGather;
-    p->slots = c.world - 1;
-    p->src0 = c.out;
-    p->block_bytes = block_bytes;
-    p->block_rows = c.M;
-    p->pitch = (uint32_t)c.ld_out_bytes;
-  } else if (c.op == tccl::kOpReduceScatter) {
-    // two ranks only: the landing slots hold one addend per rank
-    if (c.world != 2 || c.M % 2) return false;
-    const int shard = c.M / 2;
-    const int64_t block_bytes = (int64_t)shard * c.ldc_bytes;
-    if (row_bytes % 16 || c.ldc_bytes % 16 || c.ld_rs_out_bytes % 8 || block_bytes >= (int64_t)1 << 32 ||
-        (int64_t)shard * c.ld_rs_out_bytes >= (int64_t)1 << 32)
-      return false;
-    if (c.out_dtype != tccl::kF16 && c.out_dtype != tccl::kBF16) return false;
-    p->mode = tccl::kBgReduce;
-    p->emulate_peer = c.emulate_peer;
-    p->slots = c.emulate_peer ? 2 : 1;
-    p->src0 = c.C;
-    p->block_bytes = block_bytes;
-    p->block_rows = shard;
-    p->pitch = (uint32_t)c.ldc_bytes;
-    p->dst0 = c.rs_out;
-    p->dst_pitch = (uint32_t)c.ld_rs_out_bytes;
-    p->out_bf16 = c.out_dtype == tccl::kBF16;
-  } else {
-    return false;
-  }
-  p->upr = (uint32_t)(row_bytes / 16);
-  p->units = (uint32_t)p->block_rows * p->upr;
-  p->pieces = (int)((p->units + 63) / 64);
+  return true;
+}
+
+// A reduce-scatter whose reduction the large-tile kernel can perform tile by tile.
+bool build_reduce(const tccl::CommArgs& c, const tccl_sync_desc* sync, tccl::ReduceArgs* r, tccl::Macro* m) {
+  memset(r, 0, sizeof *r);
+  if (c.op != tccl::kOpReduceScatter || c.world <= 1 || c.M % c.world) return false;
+  const int shard = c.M / c.world;
+  if (shard % tccl::kMacro) return false;  // a tile must not straddle two owners
+  if (c.out_dtype != tccl::kF16 && c.out_dtype != tccl::kBF16) return false;
+  if (c.ld_rs_out_bytes % 8) return false;
+  r->active = 1;
+  r->rank = c.rank;
+  r->world = c.world;
+  r->emulate_peer = c.emulate_peer;
+  r->shard_rows = shard;
+  r->out_bf16 = c.out_dtype == tccl::kBF16;
+  r->heap_bases = c.heap_bases;
+  r->out = c.rs_out;
+  r->ld_out = c.ld_rs_out_bytes / 2;
+  r->locks = sync->locks;
+  r->counter = sync->counter;
+  r->tile_counts = sync->tile_counts;
+  r->epoch = c.epoch;
+  r->fault = c.fault;
+  r->spin_ticks = c.spin_ticks;
+  m->row_shift = ((c.rank + 1) % c.world) * (shard / tccl::kMacro);  // this rank's own rows come last
   return true;
 }
 
@@ -515,11 +526,12 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     // Pushes leave from the epilogue; what remains for the communication role are the
     // pulls (and, for a reduce-scatter, the reductions).
     if (build_push(c, g, &f.push)) c.directions &= ~tccl::kDirPush;
-    if (build_background(c, &f.pull)) {
-      if (f.pull.mode == tccl::kBgReduce)
-        c.op = tccl::kOpNone;
-      else
-        c.directions &= ~tccl::kDirPull;
+    memset(&f.reduce, 0, sizeof f.reduce);
+    if (build_reduce(c, sync, &f.reduce, &f.m)) {
+      c.op = tccl::kOpNone;
+      memset(&f.pull, 0, sizeof f.pull);
+    } else if (build_background(c, &f.pull)) {
+      c.directions &= ~tccl::kDirPull;
     }
     if (c.op != tccl::kOpReduceScatter && !(c.directions & (tccl::kDirPush | tccl::kDirPull))) c.op = tccl::kOpNone;
     f.comm = c;

@@ -61,6 +61,7 @@ struct Macro {
   int rows, cols;        // macro tile grid
   int rows_per_band;     // macro rows that form one swizzle band of the plan
   int xcds, span;        // slot -> macro id remap
+  int row_shift;         // macro rows are visited starting at this one (wrapping around)
 };
 
 // Where the epilogue sends a finished tile besides C: the same rows of every listed target,
@@ -78,40 +79,55 @@ struct PushArgs {
   const int64_t* heap_bases;  // C's address inside target q is C + heap_bases[q] - heap_bases[rank]
 };
 
-// Background transfer: the part of the collective that reads finished TileGroups of the
-// peers, carried out in the shadow of the K loop (TileGroup variant).
-//   gather (all-gather pull):  out[block of peer] <- the peer's copy of that block
-//   reduce (reduce-scatter):   out_owner[row] = cast(partial_owner[row] + partial_other[row]), two ranks
-// A block (a peer's row block / an owner's shard of the partial) is cut into pieces of 64
-// units of 16 bytes; wavefront w of the launch owns pieces w, w + W, w + 2W, ... (W =
-// wavefronts in the grid), so at any moment the grid sweeps a contiguous stretch.  Each K
-// step a wavefront finishes the piece it fetched during the previous step (store it; or add
-// the two fetched addends in fp32, round once and store) and fetches the next one straight
-// into LDS.  A piece is fetched only once the TileGroups covering its rows are complete on
-// every rank it reads from (counter[g] >= epoch * tile_counts[g], the readiness rule of
-// tileccl_v2/signal.py:43-66); that is found out by counter fetches which are themselves
-// left in flight for one K step.  What the K loops did not get to is finished after the
-// last tile, with bounded waits.  Groups must cover the rows in ascending order and not
-// straddle a block border (build_tile_group_plan with row_split_boundaries emits them so:
-// tileccl_v2/tile_group.py:156-211, 244-301).
-enum BackgroundMode { kBgNone = 0, kBgGather = 1, kBgReduce = 2 };
+// Reduce-scatter carried out tile by tile.  Once a macro tile's partial is stored and
+// published, the workgroup waits for the other ranks' partials of the same tile, streams the
+// tile back (its own copy is still in this XCD's L2), adds in fp32 -- the owner's addend
+// first, then ascending ranks; one rounding: tile_reduce_scatter, primitives/collectives.py:766-781
+// -- and writes the owner's output shard.  The accumulators are dead by then, so the stream
+// runs with many loads in flight.  Tiles are visited starting with the rows the other ranks
+// own; a rank's own rows come last, and only tiles of own rows wait on a peer (reducing on a
+// peer's behalf happens in single-GPU emulation, against resident partials).  A rank therefore
+// only ever waits for tiles its peers produce early and without waiting: no cycle.
+struct ReduceArgs {
+  int active;
+  int rank, world, emulate_peer;
+  int shard_rows;                 // rows per owner; a multiple of the 256-row tile
+  int out_bf16;                   // output element: 0 fp16, 1 bf16
+  const int64_t* heap_bases;
+  const char* out;                // the output shard in this rank's slice (the partial is the GEMM's C)
+  int64_t ld_out;                 // output pitch in elements
+  const int32_t* locks;           // this rank's words; a peer's sit at the same slice offset
+  const int32_t* counter;
+  const int32_t* tile_counts;
+  int epoch;
+  int64_t* fault;
+  int64_t spin_ticks;
+};
+
+// Background transfer: the pull half of an all-gather, carried out in the shadow of the K
+// loop (TileGroup variant): out[block of peer] <- the peer's copy of that block.
+// A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
+// pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
+// contiguous stretch.  Each K step a wavefront stores the piece it fetched during the
+// previous step and fetches the next one straight into LDS.  A piece is fetched only once
+// the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
+// tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
+// counter fetches which are themselves left in flight for one K step.  What the K loops did
+// not get to is finished after the last tile, with bounded waits.  Groups must cover the rows
+// in ascending order (build_tile_group_plan emits them so: tileccl_v2/tile_group.py:244-301).
+enum BackgroundMode { kBgNone = 0, kBgGather = 1 };
 struct PullArgs {
   int mode;
-  int slots;                   // blocks to process: gather: peers; reduce: owners handled here
+  int slots;                   // blocks to process: the peers
   int rank, world;
-  int emulate_peer;            // reduce: slot s is owner s (else the only slot is this rank's shard)
   const int64_t* heap_bases;
-  const char* src0;            // block 0 of the source in this rank's slice (gathered output / partial)
-  int64_t block_bytes;         // distance between consecutive blocks of the source (rows * pitch)
+  const char* src0;            // block 0 of the gathered output in this rank's slice
+  int64_t block_bytes;         // distance between consecutive blocks (rows * pitch)
   int block_rows;              // rows per block
-  uint32_t pitch;              // source bytes per row
-  uint32_t upr;                // 16-byte units per source row
+  uint32_t pitch;              // bytes per row
+  uint32_t upr;                // 16-byte units per row
   uint32_t units;              // units per block (rows * upr)
   int pieces;                  // pieces per block: ceil(units / 64)
-  // reduce only: the owner's output shard
-  const char* dst0;            // the output shard in this rank's slice
-  uint32_t dst_pitch;          // bytes per output row
-  int out_bf16;                // output element: 0 fp16, 1 bf16
   // synchronisation
   const int32_t* counter;      // this rank's TileGroup counters; a peer's sit at the same slice offset
   const int32_t* row_ends;
@@ -122,8 +138,8 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
 };
-constexpr int kBgPieceBytes = 8 * 2048;                 // per wavefront two 1 KiB landing slots (gather uses one)
-constexpr int kBgBytes = kBgPieceBytes + 8 * 512;       // plus two fetched counter words (64 lanes x 4 B each)
+constexpr int kBgPieceBytes = 8 * 1024;                 // one 1 KiB landing slot per wavefront
+constexpr int kBgBytes = kBgPieceBytes + 8 * 256;       // plus a fetched counter word (64 lanes x 4 B)
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
   const int per_band = m.rows_per_band * m.cols;
@@ -157,7 +173,7 @@ TCCL_D T late_kernarg(int offset) {
   return v;
 }
 
-template <typename InT, typename OutT>
+template <typename InT, typename OutT, bool kWithReduce = false>
 struct Gemm256 {
   typedef typename Mfma<InT>::Vec Vec;
   static constexpr int kEszIn = sizeof(InT);
@@ -169,7 +185,8 @@ struct Gemm256 {
 
   const GemmArgs& g;
   const PullArgs& pa;
-  const int push_offset;  // byte offset of a PushArgs in the kernel arguments; < 0: no push
+  const int push_offset;    // byte offset of a PushArgs in the kernel arguments; < 0: no push
+  const int reduce_offset;  // byte offset of a ReduceArgs in the kernel arguments; < 0: none
   // The two pipeline stages are two separate __shared__ arrays: loads that write LDS directly
   // are tracked per LDS variable, so a read of one stage need not wait for a load into the other.
   char* lds;   // stage 0 (also the epilogue's staging area)
@@ -177,9 +194,9 @@ struct Gemm256 {
   char* bg;    // landing slots of the background transfer
   const int tid, lane, wave, wm, wn;
 
-  TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, char* stage0, char* stage1,
-                 char* landing)
-      : g(args), pa(pull_args), push_offset(push_args_offset), lds(stage0), lds1(stage1), bg(landing), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+  TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, int reduce_args_offset, char* stage0,
+                 char* stage1, char* landing)
+      : g(args), pa(pull_args), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bg(landing), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
         wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
@@ -316,8 +333,8 @@ struct Gemm256 {
     int gidx;                // first TileGroup of that block not yet known complete
     int row0;                // first row of that block in the plan's row numbering
     uint32_t ready_units;    // units [0, ready_units) of that block may be fetched
-    int64_t src_base, src2_base, dst_base;  // addresses of the block in the slices involved
-    int64_t counter_base, counter2_base;    // the counter words of the ranks read from
+    int64_t src_base, dst_base;  // addresses of the block in the peer's slice and in this one
+    int64_t counter_base;        // the peer's counter words
     int probe_group;         // group whose counters were fetched during the previous step (-1: none)
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
@@ -337,13 +354,11 @@ struct Gemm256 {
     return ((const __attribute__((address_space(4))) T*)p)[i];
   }
 
-  TCCL_D bool bg_reduce() const { return pa.mode == kBgReduce; }
-
   TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
     PullState st;
     const int w = uniform(wave);
-    st.lds_off = w * 2048;
-    st.probe_off = kBgPieceBytes + w * 512;
+    st.lds_off = w * 1024;
+    st.probe_off = kBgPieceBytes + w * 256;
     st.stride = num_wgs * (kThreads256 / 64);
     st.next_slot = 0;
     st.next_lp = wg * (kThreads256 / 64) + w;
@@ -351,7 +366,7 @@ struct Gemm256 {
     st.gidx = 0;
     st.row0 = 0;
     st.ready_units = 0;
-    st.src_base = st.src2_base = st.dst_base = st.counter_base = st.counter2_base = 0;
+    st.src_base = st.dst_base = st.counter_base = 0;
     st.probe_group = -1;
     st.need = 0;
     st.group_units = 0;
@@ -378,9 +393,6 @@ struct Gemm256 {
     }
     __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter_base), (LdsVoid*)(landing + st.probe_off), 4, (uint32_t)st.gidx * 4u, 0, 0,
                                              kCoherent);
-    if (a.mode == kBgReduce)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.counter2_base), (LdsVoid*)(landing + st.probe_off + 256), 4,
-                                               (uint32_t)st.gidx * 4u, 0, 0, kCoherent);
     st.probe_group = st.gidx;
   }
 
@@ -412,34 +424,14 @@ struct Gemm256 {
     st.probe_group = -1;
     st.backoff = 0;
     const int64_t mine = table(a.heap_bases, a.rank);
-    if (a.mode == kBgGather) {
-      const int peer = slot < a.rank ? slot : slot + 1;
-      const int64_t theirs = table(a.heap_bases, peer);
-      const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)peer * a.block_bytes;
-      st.src_base = theirs + rel;
-      st.src2_base = 0;
-      st.dst_base = mine + rel;
-      st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
-      st.counter2_base = 0;
-      st.row0 = 0;  // the plan numbers the rows of one block
-      st.gidx = 0;
-      pull_group_facts(st, a);
-      return;
-    }
-    // reduce, two ranks: the owner's addend first, then the other rank's
-    const int owner = a.emulate_peer ? slot : a.rank;
-    const int other = 1 - owner;
-    const int64_t base_owner = table(a.heap_bases, owner), base_other = table(a.heap_bases, other);
-    const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)owner * a.block_bytes;
-    st.src_base = base_owner + rel;
-    st.src2_base = base_other + rel;
-    st.dst_base = base_owner + ((int64_t)(uintptr_t)a.dst0 - mine);
-    st.counter_base = (int64_t)(uintptr_t)a.counter;                  // this rank's own tiles
-    st.counter2_base = (int64_t)(uintptr_t)a.counter + (table(a.heap_bases, 1 - a.rank) - mine);
-    st.row0 = owner * a.block_rows;
-    int g = 0;
-    while (g < a.n_groups && table(a.row_ends, g) <= st.row0) ++g;  // the shard's first group
-    st.gidx = uniform(g);  // a loop's exit value does not count as uniform by itself
+    const int peer = slot < a.rank ? slot : slot + 1;
+    const int64_t theirs = table(a.heap_bases, peer);
+    const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)peer * a.block_bytes;
+    st.src_base = theirs + rel;
+    st.dst_base = mine + rel;
+    st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
+    st.row0 = 0;  // the plan numbers the rows of one block
+    st.gidx = 0;
     pull_group_facts(st, a);
   }
 
@@ -465,46 +457,13 @@ struct Gemm256 {
     }
   }
 
-  // out = cast(first + second): fp32 sum, one rounding (tile_reduce_scatter, primitives/collectives.py:766-781).
-  TCCL_D void reduce_store(const PullArgs& a, const PullState& st, u32x4 first, u32x4 second, uint32_t row, uint32_t col, bool valid) const {
-    float x[8], y[8];
-    int n;
-    unpack(first, x, n);
-    unpack(second, y, n);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] += y[e];
-    const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
-    constexpr int kElems = 16 / sizeof(OutT);
-    const uint32_t off = row * a.dst_pitch + col * (kElems * 2);
-    if constexpr (kElems == 4) {
-      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-      u32x2 w;
-      if (a.out_bf16) {
-        const __bf16 h[4] = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
-        __builtin_memcpy(&w, h, 8);
-      } else {
-        const _Float16 h[4] = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
-        __builtin_memcpy(&w, h, 8);
-      }
-      if (valid) __builtin_amdgcn_raw_buffer_store_b64(w, dst, off, 0, kStreaming);
-    } else {
-      const u32x4 w = a.out_bf16 ? pack8<__bf16>(x) : pack8<_Float16>(x);
-      if (valid) st16<kStreaming>(dst, off, w);
-    }
-  }
-
   // Finish the piece that is sitting in the landing slots.
   TCCL_D void pull_retire(PullState& st, const PullArgs& a, const char* landing) const {
     bool valid;
     uint32_t row, col;
     pull_unit(a, st.pending_lp, valid, row, col);
     const u32x4 v = *(const u32x4*)(landing + st.lds_off + lane * 16);
-    if (a.mode == kBgGather) {
-      if (valid) st16<kStreaming>(window(st.dst_base), row * a.pitch + col * 16u, v);
-    } else {
-      const u32x4 v2 = *(const u32x4*)(landing + st.lds_off + 1024 + lane * 16);
-      reduce_store(a, st, v, v2, row, col, valid);
-    }
+    if (valid) st16<kStreaming>(window(st.dst_base), row * a.pitch + col * 16u, v);
     st.pending_lp = -1;
   }
 
@@ -529,11 +488,7 @@ struct Gemm256 {
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
       st.probe_group = -1;
-      int32_t seen = uniform(*(const int32_t*)(landing + st.probe_off));
-      if (a.mode == kBgReduce) {
-        const int32_t seen2 = uniform(*(const int32_t*)(landing + st.probe_off + 256));
-        seen = seen2 < seen ? seen2 : seen;
-      }
+      const int32_t seen = uniform(*(const int32_t*)(landing + st.probe_off));
       if (g == st.gidx) {
         if (seen >= st.need)
           pull_group_done(st, a);
@@ -553,8 +508,6 @@ struct Gemm256 {
       pull_unit(a, st.next_lp, valid, row, col);
       const uint32_t off = row * a.pitch + col * 16u;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(landing + st.lds_off), 16, off, 0, 0, kCoherent);
-      if (a.mode == kBgReduce)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src2_base), (LdsVoid*)(landing + st.lds_off + 1024), 16, off, 0, 0, kCoherent);
       st.pending_lp = st.next_lp;
       st.next_lp += st.stride;
       pull_normalise(st, a);
@@ -568,11 +521,9 @@ struct Gemm256 {
       if (st.gidx >= a.n_groups) return false;
       const int32_t need = st.need;
       const __amdgpu_buffer_rsrc_t words = window(st.counter_base);
-      const __amdgpu_buffer_rsrc_t words2 = window(a.mode == kBgReduce ? st.counter2_base : st.counter_base);
       for (;;) {
         const int32_t seen = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(words, (uint32_t)st.gidx * 4u, 0, kCoherent);
-        const int32_t seen2 = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(words2, (uint32_t)st.gidx * 4u, 0, kCoherent);
-        if (uniform(seen) >= need && uniform(seen2) >= need) break;
+        if (uniform(seen) >= need) break;
         if (now_ticks() > deadline) return false;
         __builtin_amdgcn_s_sleep(8);
       }
@@ -592,7 +543,7 @@ struct Gemm256 {
     constexpr int kBatch = 8;  // pieces in flight per wavefront: the CU has no other work left
     while (ok && st.next_slot < a.slots) {
       pull_select(st, a, st.next_slot);
-      u32x4 v[kBatch], v2[kBatch];
+      u32x4 v[kBatch];
       uint32_t row[kBatch], col[kBatch];
       bool valid[kBatch], loaded[kBatch];
       int n = 0;
@@ -606,7 +557,6 @@ struct Gemm256 {
             pull_unit(a, lp, valid[k], row[k], col[k]);
             const uint32_t off = row[k] * a.pitch + col[k] * 16u;
             v[k] = ld16<kCoherent>(window(st.src_base), off);
-            if (a.mode == kBgReduce) v2[k] = ld16<kCoherent>(window(st.src2_base), off);
             loaded[k] = true;
             n = k + 1;
           }
@@ -614,12 +564,7 @@ struct Gemm256 {
       }
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
-        if (!loaded[k]) continue;
-        if (a.mode == kBgGather) {
-          if (valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a.pitch + col[k] * 16u, v[k]);
-        } else {
-          reduce_store(a, st, v[k], v2[k], row[k], col[k], valid[k]);
-        }
+        if (loaded[k] && valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a.pitch + col[k] * 16u, v[k]);
       }
       st.next_lp += n * st.stride;
       if (n < kBatch) {  // the block is finished (or a wait gave up)
@@ -806,6 +751,127 @@ struct Gemm256 {
       wait_vmem();  // the tile's write-through stores have landed
       __syncthreads();
       if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+      if constexpr (kWithReduce) {
+        const ReducePtr ra = late_kernarg_ptr<ReduceArgs>(reduce_offset);
+        if (ra->active) {
+          const int owner = row0 / ra->shard_rows;
+          if ((owner == ra->rank || ra->emulate_peer) && reduce_wait(ra, s, mm, mn)) reduce_tile(ra, row0, col0, owner);
+        }
+      }
+    }
+  }
+
+  typedef const __attribute__((address_space(4))) ReduceArgs* ReducePtr;
+
+  // Are the peers' partials of the plan tiles under macro tile (mm, mn) published?  One lane
+  // waits (bounded); the verdict travels through an LDS word of the idle stage.
+  TCCL_D bool reduce_wait(ReducePtr ra, const SignalArgs& s, int mm, int mn) const {
+    volatile int* verdict = (volatile int*)lds1;
+    if (tid == 0) {
+      bool ok = true;
+      const int64_t deadline = now_ticks() + ra->spin_ticks;
+      const int64_t mine = ra->heap_bases[ra->rank];
+      const int tm0 = mm * (kMacro / g.block_m), tn0 = mn * (kMacro / g.block_n);
+      for (int p = 0; p < ra->world && ok; ++p) {
+        if (p == ra->rank) continue;
+        const int64_t delta = ra->heap_bases[p] - mine;
+        int waited_group = -1;
+        for (int dm = 0; dm < kMacro / g.block_m && ok; ++dm)
+          for (int dn = 0; dn < kMacro / g.block_n && ok; ++dn) {
+            const int tm = tm0 + dm, tn = tn0 + dn;
+            if (tm >= g.tile_rows || tn >= g.tile_cols) continue;
+            const int tile_id = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
+            if (s.mode == kSignalTile) {
+              ok = tile_wait<true>((int32_t*)((char*)ra->locks + delta), tile_id, /*consume=*/false, deadline);
+            } else {
+              const int gi = s.group_table[tile_id];
+              if (gi == waited_group) continue;
+              waited_group = gi;
+              ok = tile_wait_ge<true>((const int32_t*)((const char*)ra->counter + delta), gi, ra->epoch * ra->tile_counts[gi], deadline);
+            }
+          }
+      }
+      if (!ok && ra->fault) *ra->fault = 1;
+      *verdict = ok ? 1 : 0;
+    }
+    __syncthreads();
+    const bool all_ok = *verdict != 0;
+    __syncthreads();
+    return all_ok;
+  }
+
+  // out_owner[tile] = cast(sum over ranks of partial_rank[tile]); the whole workgroup streams
+  // the tile in 16-byte units, kUnroll units per thread in flight.
+  TCCL_D void reduce_tile(ReducePtr ra, int row0, int col0, int owner) const {
+    constexpr int kEsz = sizeof(OutT);
+    constexpr int kE = 16 / kEsz;
+    constexpr int kUnroll = 4;
+    const int rows = g.M - row0 < kMacro ? g.M - row0 : kMacro;
+    const int cols = g.N - col0 < kMacro ? g.N - col0 : kMacro;
+    const int upr = cols / kE;  // N is a multiple of 8, so a row holds whole units
+    const int total = rows * upr;
+    const int world = ra->world, rank = ra->rank;
+    const int64_t my_base = ra->heap_bases[rank];
+    const int64_t tile_off = ((int64_t)row0 * g.ldc + col0) * kEsz;
+    const int64_t ld_out = ra->ld_out;
+    const __amdgpu_buffer_rsrc_t r_mine = window((int64_t)(uintptr_t)g.C + tile_off);
+    const __amdgpu_buffer_rsrc_t r_out = window((int64_t)(uintptr_t)ra->out + (ra->heap_bases[owner] - my_base) +
+                                                ((int64_t)(row0 - owner * ra->shard_rows) * ld_out + col0) * 2);
+    const bool bf = ra->out_bf16 != 0;
+    for (int u0 = tid; u0 < total; u0 += kThreads256 * kUnroll) {
+      u32x4 mine[kUnroll];
+      uint32_t src[kUnroll], dst[kUnroll];
+      bool live[kUnroll];
+      float sum[kUnroll][8];
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int u = u0 + k * kThreads256;
+        live[k] = u < total;
+        const uint32_t uu = live[k] ? (uint32_t)u : 0u;  // idle lanes re-read the first unit and store nothing
+        const uint32_t r = uu / (uint32_t)upr, c = uu - r * (uint32_t)upr;
+        src[k] = (uint32_t)((r * g.ldc + c * kE) * kEsz);
+        dst[k] = (uint32_t)((r * ld_out + c * kE) * 2);
+        mine[k] = ld16<0>(r_mine, src[k]);  // this workgroup just wrote it: served by this XCD's L2
+      }
+      for (int step = 0; step < world; ++step) {
+        // owner first, then the other ranks in ascending order
+        const int p = step == 0 ? owner : (step - 1 < owner ? step - 1 : step);
+        u32x4 addend[kUnroll];
+        if (p == rank) {
+#pragma unroll
+          for (int k = 0; k < kUnroll; ++k) addend[k] = mine[k];
+        } else {
+          const __amdgpu_buffer_rsrc_t r_peer = window((int64_t)(uintptr_t)g.C + (ra->heap_bases[p] - my_base) + tile_off);
+#pragma unroll
+          for (int k = 0; k < kUnroll; ++k) addend[k] = ld16<kCoherent>(r_peer, src[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+          float f[8];
+          int n;
+          unpack(addend[k], f, n);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sum[k][e] = step == 0 ? f[e] : sum[k][e] + f[e];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        if constexpr (kE == 4) {
+          typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+          u32x2 o;
+          if (bf) {
+            const __bf16 h[4] = {(__bf16)sum[k][0], (__bf16)sum[k][1], (__bf16)sum[k][2], (__bf16)sum[k][3]};
+            __builtin_memcpy(&o, h, 8);
+          } else {
+            const _Float16 h[4] = {(_Float16)sum[k][0], (_Float16)sum[k][1], (_Float16)sum[k][2], (_Float16)sum[k][3]};
+            __builtin_memcpy(&o, h, 8);
+          }
+          if (live[k]) __builtin_amdgcn_raw_buffer_store_b64(o, r_out, dst[k], 0, kStreaming);
+        } else {
+          const u32x4 o = bf ? pack8<__bf16>(sum[k]) : pack8<_Float16>(sum[k]);
+          if (live[k]) st16<kStreaming>(r_out, dst[k], o);
+        }
+      }
     }
   }
 
@@ -845,7 +911,9 @@ struct Gemm256 {
     pull_prime(pull, pa, bg);
     for (int slot = wg; slot < total; slot += num_wgs) {
       const int id = tile_for_slot(slot, total, m.xcds, m.span);
-      const TileCoord c = macro_coords(id, m);
+      TileCoord c = macro_coords(id, m);
+      c.m += m.row_shift;
+      if (c.m >= m.rows) c.m -= m.rows;
       if (s.mode == kSignalNone && push_offset < 0)
         macro_tile<0>(s, c.m, c.n, pull);
       else
