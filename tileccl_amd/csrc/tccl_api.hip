@@ -349,6 +349,9 @@ tccl::Macro build_macro(const tccl_gemm_desc* d, const tccl_device_info& dev, in
 int default_macro_wgs(const tccl_gemm_desc* d, const tccl_device_info& dev) {
   const int total = ((d->M + 255) / 256) * ((d->N + 255) / 256);
   int n = d->num_wgs > 0 ? d->num_wgs : dev.compute_units;
+  // One workgroup fills a CU, and workgroups of a fused launch wait on each other's tiles
+  // after their own: every workgroup must be resident, so the grid never exceeds the CUs.
+  if (n > dev.compute_units) n = dev.compute_units;
   if (n > total) n = total;
   return n < 1 ? 1 : n;
 }

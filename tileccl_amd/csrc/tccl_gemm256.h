@@ -108,8 +108,9 @@ struct ReduceArgs {
 // loop (TileGroup variant): out[block of peer] <- the peer's copy of that block.
 // A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
 // pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
-// contiguous stretch.  Each K step a wavefront stores the piece it fetched during the
-// previous step and fetches the next one straight into LDS.  A piece is fetched only once
+// contiguous stretch.  At the start of a K step a wavefront fetches its next piece straight
+// into one of its two LDS landing slots; at the end of the step, behind the MFMAs, it stores
+// the piece the previous step fetched.  A piece is fetched only once
 // the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
 // tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
 // counter fetches which are themselves left in flight for one K step.  What the K loops did
@@ -138,7 +139,7 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
 };
-constexpr int kBgPieceBytes = 8 * 1024;                 // one 1 KiB landing slot per wavefront
+constexpr int kBgPieceBytes = 8 * 2048;                 // two 1 KiB landing slots per wavefront (alternating K steps)
 constexpr int kBgBytes = kBgPieceBytes + 8 * 256;       // plus a fetched counter word (64 lanes x 4 B)
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
@@ -339,7 +340,8 @@ struct Gemm256 {
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
-    int pending_lp;          // piece fetched into LDS during the previous step (-1: none)
+    int pending_lp[2];       // per landing slot: the piece fetched into it and not yet stored (-1: none)
+    int64_t pending_dst[2];  // and the destination block's address
     int lds_off;             // this wavefront's landing slots inside the landing array
     int probe_off;           // and its counter landing words
   };
@@ -357,7 +359,7 @@ struct Gemm256 {
   TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
     PullState st;
     const int w = uniform(wave);
-    st.lds_off = w * 1024;
+    st.lds_off = w * 2048;
     st.probe_off = kBgPieceBytes + w * 256;
     st.stride = num_wgs * (kThreads256 / 64);
     st.next_slot = 0;
@@ -371,7 +373,8 @@ struct Gemm256 {
     st.need = 0;
     st.group_units = 0;
     st.backoff = 0;
-    st.pending_lp = -1;
+    st.pending_lp[0] = st.pending_lp[1] = -1;
+    st.pending_dst[0] = st.pending_dst[1] = 0;
     if (a.mode != kBgNone) pull_normalise(st, a);
     return st;
   }
@@ -457,14 +460,20 @@ struct Gemm256 {
     }
   }
 
-  // Finish the piece that is sitting in the landing slots.
-  TCCL_D void pull_retire(PullState& st, const PullArgs& a, const char* landing) const {
+  // Store the piece sitting in landing slot `slot`, if any.  Returns whether a store was issued.
+  TCCL_D bool pull_retire(PullState& st, const PullArgs& a, const char* landing, int slot) const {
+    if (a.mode == kBgNone || st.pending_lp[slot] < 0) return false;
     bool valid;
     uint32_t row, col;
-    pull_unit(a, st.pending_lp, valid, row, col);
-    const u32x4 v = *(const u32x4*)(landing + st.lds_off + lane * 16);
-    if (valid) st16<kStreaming>(window(st.dst_base), row * a.pitch + col * 16u, v);
-    st.pending_lp = -1;
+    pull_unit(a, st.pending_lp[slot], valid, row, col);
+    const u32x4 v = *(const u32x4*)(landing + st.lds_off + slot * 1024 + lane * 16);
+    // The store must use the bases of the block the piece belongs to: pieces are retired
+    // before the slot selection moves on (pull_issue), except for the one in flight when it
+    // does, whose bases are kept aside.
+    const int64_t dst = st.pending_dst[slot];
+    if (valid) st16<kStreaming>(window(dst), row * a.pitch + col * 16u, v);
+    st.pending_lp[slot] = -1;
+    return true;
   }
 
   // The two facts about group gidx that the per-step code needs, fetched when gidx changes.
@@ -479,12 +488,11 @@ struct Gemm256 {
     pull_group_facts(st, a);
   }
 
-  // The per-K-step slice of the transfer; all control flow here is wavefront-uniform.  One
-  // landing array serves every step: a slot is read back (and the read waited for) before
-  // the next fetch into it is issued, and the fetch has landed by the step's closing wait.
-  TCCL_D void pull_step(PullState& st, const PullArgs& a, char* landing) const {
+  // Start of a K step: learn about readiness, fetch the next piece into landing slot `slot`
+  // (its previous piece was stored at the end of the step before last).  All control flow
+  // here is wavefront-uniform.
+  TCCL_D void pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
     if (a.mode == kBgNone) return;
-    if (st.pending_lp >= 0) pull_retire(st, a, landing);
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
       st.probe_group = -1;
@@ -507,8 +515,10 @@ struct Gemm256 {
       uint32_t row, col;
       pull_unit(a, st.next_lp, valid, row, col);
       const uint32_t off = row * a.pitch + col * 16u;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(landing + st.lds_off), 16, off, 0, 0, kCoherent);
-      st.pending_lp = st.next_lp;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(landing + st.lds_off + slot * 1024), 16, off, 0, 0,
+                                               kCoherent);
+      st.pending_lp[slot] = st.next_lp;
+      st.pending_dst[slot] = st.dst_base;
       st.next_lp += st.stride;
       pull_normalise(st, a);
     }
@@ -536,7 +546,8 @@ struct Gemm256 {
   TCCL_D void pull_finish(PullState& st, const PullArgs& a, const char* landing, int num_wgs) const {
     if (a.mode == kBgNone) return;
     wait_vmem();
-    if (st.pending_lp >= 0) pull_retire(st, a, landing);
+    pull_retire(st, a, landing, 0);
+    pull_retire(st, a, landing, 1);
     st.probe_group = -1;
     const int64_t deadline = now_ticks() + a.spin_ticks;
     bool ok = true;
@@ -596,9 +607,10 @@ struct Gemm256 {
   // MFMAs; holding a second fragment set would push the kernel past 256 registers and the
   // spill reloads would drain the load queue every step.  The scheduling barrier keeps the
   // compiler from hoisting the next chunk's reads across the MFMAs.
-  TCCL_D void k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
-                     PullState& pull) const {
-    pull_step(pull, pa, bg);
+  // Returns whether the step ended with a background store (the youngest memory operation).
+  TCCL_D bool k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
+                     PullState& pull, int parity) const {
+    pull_issue(pull, pa, bg, parity);
     if constexpr (kFp8) {
       // An fp8 operand is 8 registers: the A slabs are fetched one at a time so that the
       // fragments in flight stay within what the 16-bit path holds.
@@ -643,6 +655,23 @@ struct Gemm256 {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    return pull_retire(pull, pa, bg, parity ^ 1);  // behind the MFMAs: the piece the previous step fetched
+  }
+
+  // Close a step: this wave's loads into the next stage (and its background fetch) have
+  // landed; a background store issued at the very end may stay in flight.  The barrier is the
+  // bare instruction: __syncthreads() carries a workgroup-scope release fence, which on this
+  // target waits for vmcnt(0) and would wait for that store too.  What must be ordered is
+  // ordered by hand: the loads have landed (the wait), and this wave's LDS reads of the stage
+  // about to be overwritten fed MFMAs that are already issued.  The empty asm keeps the
+  // compiler from moving LDS accesses across the barrier.
+  TCCL_D void close_step(bool stored) const {
+    if (stored)
+      asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   }
 
   // Stores the tile and, when a push is asked for, sends it to the peers from the same LDS staging.
@@ -739,12 +768,8 @@ struct Gemm256 {
     wait_vmem();
     __syncthreads();
     for (int kt = 0; kt < ksteps; kt += 2) {
-      k_step(lds, lds1, src, rd, kt + 1, acc, pull);
-      wait_vmem();
-      __syncthreads();
-      k_step(lds1, lds, src, rd, kt + 2, acc, pull);
-      wait_vmem();
-      __syncthreads();
+      close_step(k_step(lds, lds1, src, rd, kt + 1, acc, pull, 0));
+      close_step(k_step(lds1, lds, src, rd, kt + 2, acc, pull, 1));
     }
     epilogue<kPolicy>(row0, col0, acc);
     if constexpr (kPolicy != 0) {
