@@ -105,3 +105,43 @@ def test_fp8_reduce_scatter_two_ranks(lib, variant):
     finally:
         for h in heaps:
             h.cleanup()
+
+
+def test_baseline_config_4_properties(lib):
+    """16384x2048 @ 2048x4096 e4m3 with per-tensor scales, resident bf16 peer partial: the three
+    variants agree byte for byte, the reduction equals the oracle on slabs of both owners, the
+    partial matches the dequantised matmul on a slab, counters match the plan."""
+    from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
+
+    M, N, K = 16384, 4096, 2048
+    heaps = SymmetricHeap.create_all(1 << 30, 2)
+    try:
+        ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=torch.bfloat16, out_dtype=torch.bfloat16) for h in heaps]
+        op = ops[0]
+        assert op.plan.n_groups == 16 and op.shard_rows == 8192
+        A_cpu, sa = quantise((M, K), 0)
+        B_cpu, sb = quantise((K, N), 1, K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        g = torch.Generator(device="cuda").manual_seed(2)
+        ops[1].partial.copy_(torch.randn(M, N, generator=g, device="cuda").bfloat16())
+        outs = {}
+        for variant in ("s0", "s1", "s2"):
+            for o in ops:
+                o.out.zero_()
+            op.mark_peers_ready()
+            op(A, B, variant, scale_a=sa, scale_b=sb)
+            op.check_faults()
+            outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
+        for v in ("s1", "s2"):
+            assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
+        for owner in (0, 1):
+            rows = slice(owner * 8192 + 100, owner * 8192 + 228)
+            want = (op.partial[rows].float() + ops[1].partial[rows].float()).bfloat16()
+            assert torch.equal(bits(outs["s2"][owner][100:228]), bits(want))
+        rows = slice(8100, 8228)
+        ref = (A_cpu[rows].float() @ B_cpu.float()) * (sa * sb)
+        assert_gemm_close(op.partial[rows], ref, rtol=5e-2, tight=0.032)
+        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+    finally:
+        for h in heaps:
+            h.cleanup()
