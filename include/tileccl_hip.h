@@ -98,7 +98,7 @@ typedef struct tccl_gemm_desc {
  *   locks      int32[total_tiles]   S1: tile_signal / tile_wait (sync/primitives.py:357-414)
  *   group_table int32[total_tiles]  S2: swizzled tile id -> group id (tile_group.py:214-241)
  *   counter    int32[n_groups]      S2: tile_signal_add / tile_wait_ge (tileccl_v2/ipc.py:231-254)
- *   barrier    int32[n_groups]      S2: finished communication tasks per group
+ *   barrier    int32[n_groups]      S2: finished communication tasks (or workgroups, see below) per group
  *   trace_*    optional device-clock stamps (signal.py:18-24); NULL to skip
  * locks, counter and barrier live in the symmetric heap, so a peer's copy sits at the
  * same offset in the peer's slice.  The host zeroes them before a launch
@@ -214,7 +214,14 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
  *             wait per tile (WGSpecializedPattern, wg_specialized.py:212-352).
  * variant S2: one launch; GEMM workgroups add to counter[group_table[tile]];
  *             communication workgroups wait per TileGroup and move copy_elems-sized
- *             tasks (reference README.md:66-84; contract in tileccl_v2/*.py). */
+ *             tasks (reference README.md:66-84; contract in tileccl_v2/*.py).
+ * With the 256 x 256 GEMM tile (gemm->macro_tile) S1 and S2 are still one launch, but a
+ * workgroup fills its CU, so the communication is done by the GEMM workgroups themselves:
+ * pushes leave from the epilogue, all-gather pulls run inside the K loop (S2) or after the
+ * workgroup's last tile (S1), reduce-scatter tiles are reduced right after they are
+ * published.  barrier[g] then advances by the grid size per launch, not by the task count.
+ * Every device-side wait is bounded by sync->spin_limit_ns; an expired wait sets *sync->fault
+ * and the kernel still runs to its end. */
 
 /* tileccl.ops.gemm_allscatter (ops.py:810-888): C = A@B locally, then the rank's column
  * block is stored into every peer's C. */
