@@ -12,12 +12,16 @@
 // LDS layout is fixed to "lanes in order" and the swizzle that keeps the MFMA reads free of
 // bank conflicts is applied on the global side, by choosing which 16-byte chunk a lane
 // fetches:
-//   A stage: row-major, 128 B per row (64 k); chunk kc of row r lives in slot kc ^ ((r >> 1) & 7).
-//   B stage: natural [k][n], 512 B per k row; chunk c of row k lives in slot c ^ (4 * (k & 3)).
-// A operands are read with ds_read_b128 (8 consecutive k of one row).  B operands are read
-// with ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of 4 consecutive n of
-// k row i/4 at column block i%4, and lane j receives 4 consecutive k for column j; two reads
-// give a lane the 8 consecutive k of v_mfma_f32_32x32x16.
+//   A stage: row-major, 128 B per row (64 k of a 16-bit type, 128 k of fp8); chunk kc of row r
+//            lives in slot kc ^ ((r >> 1) & 7).
+//   B stage: natural [k][n]; 16-bit: 512 B per k row, chunk c of row k in slot c ^ (4 * (k & 3));
+//            fp8: 256 B per k row, chunk c of row k in slot c ^ (2 * (k & 7)).
+// A operands are read with ds_read_b128.  B operands are read with the transposing LDS reads
+// of gfx950 (semantics measured on the device, 16 lanes at a time):
+//   ds_read_b64_tr_b16: lane i supplies 4 consecutive n of k row i/4 at column block i%4; lane j
+//                       receives 4 consecutive k of column j (two reads = the 8 k of 32x32x16);
+//   ds_read_b64_tr_b8:  lane i supplies 8 consecutive n of k row i/2 at column block i%2; lane j
+//                       receives 8 consecutive k of column j (four reads = the 32 k of 32x32x64).
 //
 // Pipeline: LDS holds two stages.  The loads of step kt+1 are issued, woven between the
 // MFMAs of step kt, into the stage step kt-1 has just left; `s_waitcnt vmcnt(0)` and one
@@ -81,7 +85,7 @@ struct PushArgs {
 
 // Reduce-scatter carried out tile by tile.  Once a macro tile's partial is stored and
 // published, the workgroup waits for the other ranks' partials of the same tile, streams the
-// tile back (its own copy is still in this XCD's L2), adds in fp32 -- the owner's addend
+// tile back, adds in fp32 -- the owner's addend
 // first, then ascending ranks; one rounding: tile_reduce_scatter, primitives/collectives.py:766-781
 // -- and writes the owner's output shard.  The accumulators are dead by then, so the stream
 // runs with many loads in flight.  Tiles are visited starting with the rows the other ranks
@@ -602,11 +606,7 @@ struct Gemm256 {
   }
 
   // One K step: the MFMAs of this step run from `cur` while the next step's operands
-  // stream into `nxt`, one A piece and one B piece per k-chunk.  Fragments are single
-  // buffered: two waves share a SIMD, so while one waits for its LDS reads the other issues
-  // MFMAs; holding a second fragment set would push the kernel past 256 registers and the
-  // spill reloads would drain the load queue every step.  The scheduling barrier keeps the
-  // compiler from hoisting the next chunk's reads across the MFMAs.
+  // stream into `nxt`, one A piece and one B piece per k-block.
   // Returns whether the step ended with a background store (the youngest memory operation).
   TCCL_D bool k_step(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                      PullState& pull, int parity) const {
@@ -856,7 +856,7 @@ struct Gemm256 {
         const uint32_t r = uu / (uint32_t)upr, c = uu - r * (uint32_t)upr;
         src[k] = (uint32_t)((r * g.ldc + c * kE) * kEsz);
         dst[k] = (uint32_t)((r * ld_out + c * kE) * 2);
-        mine[k] = ld16<0>(r_mine, src[k]);  // this workgroup just wrote it: served by this XCD's L2
+        mine[k] = ld16<0>(r_mine, src[k]);  // written by this workgroup itself: a plain load sees it
       }
       for (int step = 0; step < world; ++step) {
         // owner first, then the other ranks in ascending order
