@@ -38,6 +38,8 @@ WORKLOADS = {
     "c2_256": ("ag", 8192, 4096, 1024, 256, "f16"),
     "c3": ("rs", 8192, 4096, 2048, 128, "f16"),
     "c4": ("rs", 16384, 4096, 2048, 128, "f8"),
+    # gather -> GEMM -> scatter over column shards of the input (K = 2 shards of 1024)
+    "ch1": ("ch", 4096, 4096, 2048, 128, "f16"),
 }
 METRIC = "fused GEMM+AllGather ms & TFLOP/s (MFMA util), 8192x4096x1024 fp16, 1 GPU"
 
@@ -190,6 +192,105 @@ class Workload:
             h.cleanup()
 
 
+class ChainedWorkload:
+    """AllGather -> GEMM -> scatter (ChainedAGGemmRSPattern) with the interface of Workload."""
+
+    SCHEDULES = {"s0": "bulk_sync", "s1": "wg_specialized", "s2": "tile_group"}
+
+    def __init__(self, name, macro_tile):
+        import torch
+
+        import tileccl_amd as tileccl
+        from tileccl_amd.patterns.chained_ag_gemm_rs import ChainedAGGemmRSPattern
+
+        self.name = name
+        self.kind, self.M, self.N, self.K, self.block_m, self.in_type = WORKLOADS[name]
+        M, N, K = self.M, self.N, self.K
+        self.ctxs = tileccl.init_local(world_size=2, heap_size=1 << 30)
+        ks = K // 2
+        self.shards_cpu = [seeded((M, ks), 10 + p) for p in range(2)]
+        self.W_cpu = seeded((K, N), 1, K**-0.5)
+        self.shards, self.outs = [], []
+        for c, sc in zip(self.ctxs, self.shards_cpu):
+            t = c.zeros(M, ks, dtype=torch.float16)
+            t.copy_(sc)
+            self.shards.append(t)
+            self.outs.append(c.zeros(M, N, dtype=torch.float16))
+        self.W = self.ctxs[0].zeros(K, N, dtype=torch.float16)
+        self.W.copy_(self.W_cpu)
+        self.patterns = {v: ChainedAGGemmRSPattern(self.ctxs[0], schedule=sch) for v, sch in self.SCHEDULES.items()}
+        self.last = None
+        self.macro_tile = macro_tile
+        self.flop = 2.0 * M * N * K
+        # gather: both shards read, the gathered input written; scatter: the output read and written once more
+        self.exchange_bytes = 2.0 * M * K * 2 + 2.0 * M * N * 2
+
+    # main() reads these through `w.op`
+    @property
+    def op(self):
+        return self
+
+    @property
+    def plan(self):
+        return self.patterns["s2"]._stage.last_plan
+
+    def check_faults(self):
+        if self.last is not None:
+            self.last.check_faults()
+
+    def run(self, variant):
+        self.last = self.patterns[variant]
+        self.last.execute(self.shards[0], self.W, self.outs[0])
+
+    def describe(self, variant):
+        M, N, K = self.M, self.N, self.K
+        return (f"{self.name}: AllGather -> GEMM -> scatter, 2 column shards {M}x{K // 2} fp16 -> {M}x{K} @ {K}x{N}, "
+                f"output stored to both emulated heap slices, schedule {self.SCHEDULES[variant]}")
+
+    def spot_check(self):
+        import torch
+
+        from oracle import collectives as oracle
+
+        M, K = self.M, self.K
+        gathered = self.ctxs[0].workspace("chained_ag_gemm_rs.gathered_input", M, K, dtype=torch.float16)
+        assert torch.equal(gathered.cpu().view(torch.int16), oracle.gather_cols(self.shards_cpu).view(torch.int16))
+        assert torch.equal(self.outs[0].view(torch.int16), self.outs[1].view(torch.int16))
+        want = oracle.gather_cols([s[:256] for s in self.shards_cpu]).float() @ self.W_cpu.float()
+        assert torch.allclose(self.outs[0][:256].float().cpu(), want, rtol=1e-2, atol=1e-1)
+
+    def gemm_only(self):
+        import ctypes as C
+
+        import torch
+
+        from tileccl_amd import _launch, _lib
+
+        gathered = self.ctxs[0].workspace("chained_ag_gemm_rs.gathered_input", self.M, self.K, dtype=torch.float16)
+        desc = _launch.gemm_desc(gathered, self.W, self.outs[0], block_m=self.block_m, macro_tile=self.macro_tile)
+        lib = _lib.load()
+        return lambda _variant: _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
+
+    def cpu_baseline(self, iters=3):
+        import torch
+
+        from oracle import collectives as oracle
+
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        best = float("inf")
+        for _ in range(iters):
+            outs = [torch.zeros(self.M, self.N, dtype=torch.float16) for _ in range(2)]
+            t0 = time.perf_counter()
+            oracle.chained_ag_gemm_rs(self.shards_cpu, self.W_cpu, outs, 0)
+            best = min(best, time.perf_counter() - t0)
+        return best, cores
+
+    def close(self):
+        for c in self.ctxs:
+            c.heap.cleanup()
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -212,7 +313,7 @@ def main() -> int:
 
     _lib.load()
     props = get_backend().get_device_properties()
-    w = Workload(args.workload, args.macro_tile)
+    w = (ChainedWorkload if WORKLOADS[args.workload][0] == "ch" else Workload)(args.workload, args.macro_tile)
 
     results = {}
     wanted = [v for v in ("s0", "s1", "s2") if v in args.variants.split(",") or v == args.variant]

@@ -198,6 +198,14 @@ int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes,
  * slice; rank r's block occupies rows [r*rows_per_rank, (r+1)*rows_per_rank). */
 int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, int32_t elem_bytes,
                        const tccl_heap_view* heap, const tccl_transport_desc* transport, void* stream);
+/* tccl_gather_cols: the gather worker of ChainedAGGemmRSPattern
+ * (patterns/chained_ag_gemm_rs.py:262-340).  Every rank holds an M x cols `shard` at the same
+ * heap offset; column block p of this rank's `gathered` (M x world*cols, leading dim
+ * ld_gathered, in its slice) receives rank p's shard: the own one by a local copy, the
+ * others by remote loads. */
+int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int64_t ld_shard, int32_t M,
+                     int32_t cols, int32_t elem_bytes, const tccl_heap_view* heap,
+                     const tccl_transport_desc* transport, void* stream);
 /* tccl_reduce_rows: pull-reduce of tile_reduce_scatter (collectives.py:730-783) over row
  * shards with fp32 accumulation: out[r - row_lo] = cast(sum_p partial_p[r]) for
  * r in [row_lo, row_hi), where partial_p is `partial` translated into slice p, summed
@@ -228,6 +236,16 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
 int tccl_gemm_allscatter(const tccl_gemm_desc* gemm, const tccl_scatter_desc* scatter,
                          const tccl_heap_view* heap, const tccl_sync_desc* sync,
                          const tccl_transport_desc* transport, int32_t variant, void* stream);
+
+/* ChainedAGGemmRSPattern.execute (patterns/chained_ag_gemm_rs.py:120-200): gather the ranks'
+ * column shards of the input into gemm->A (M x K, K = world * k_shard, in this rank's slice),
+ * output = gathered @ W (gemm->B), and store every output tile into every peer's output at
+ * the same offset (scatter worker, :393-425).  The gather is one bulk launch ahead of the
+ * GEMM; `variant` selects how the GEMM and the stores to the peers overlap (S0: GEMM kernel,
+ * then a copy kernel; S1/S2: one launch, as tccl_gemm_allscatter). */
+int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* gemm, const void* shard, int64_t ld_shard, int32_t k_shard,
+                            const tccl_heap_view* heap, const tccl_sync_desc* sync,
+                            const tccl_transport_desc* transport, int32_t variant, void* stream);
 
 /* GEMM-output AllGather (Gate 1).  gemm->C must point at row rank*M of `out`. */
 int tccl_gemm_allgather(const tccl_gemm_desc* gemm, void* out, int64_t ld_out,

@@ -13,6 +13,9 @@ All arithmetic is torch on the CPU.  Follows
         /root/reference/tileccl/primitives/collectives.py:766-783
     (this build accumulates the reduction in fp32 and rounds once, as its north star asks;
      the reference accumulates in the tensor dtype)
+    chained gather -> GEMM -> scatter: column block p of the gathered input is rank p's shard
+        /root/reference/tileccl/patterns/chained_ag_gemm_rs.py:262-340 (gather), :343-391 (GEMM),
+        :393-425 (every tile stored to every peer)
 """
 
 from __future__ import annotations
@@ -102,6 +105,27 @@ def gemm_reducescatter(A, B, partials, outs, rank: int, emulate_peer: bool = Tru
     for owner in range(len(partials)):
         if owner == rank or emulate_peer:
             outs[owner].copy_(reduce_rows(partials, owner, outs[owner].dtype))
+
+
+def gather_cols(shards) -> torch.Tensor:
+    """Gathered input: shard p occupies columns [p*K_shard, (p+1)*K_shard) (chained_ag_gemm_rs.py:270-337).
+
+    The reference kernel offsets workspace rows by the column stride (:298, :353), which makes
+    rows overlap; this follows the layout its docstring and its (M, K) workspace state."""
+    M, ks = shards[0].shape
+    out = torch.empty(M, ks * len(shards), dtype=shards[0].dtype)
+    for p, s in enumerate(shards):
+        out[:, p * ks : (p + 1) * ks] = s
+    return out
+
+
+def chained_ag_gemm_rs(shards, W, outs, rank: int, alpha: float = 1.0) -> torch.Tensor:
+    """outs[q] = gather_cols(shards) @ W for every rank q (rank ``rank`` computes, all receive).  Returns the gathered input."""
+    gathered = gather_cols(shards)
+    result = gemm(gathered, W, outs[rank].dtype, alpha)
+    for o in outs:
+        o.copy_(result)
+    return gathered
 
 
 def expected_counters(tile_counts, epoch: int = 1):

@@ -22,7 +22,7 @@ def test_every_declared_symbol_is_exported_and_typed(lib):
     from tileccl_amd import _lib
 
     names = declared_functions()
-    assert len(names) >= 19 and "tccl_gemm_allgather" in names
+    assert len(names) >= 21 and "tccl_gemm_allgather" in names and "tccl_chained_ag_gemm_rs" in names
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names  # the ctypes table covers the header exactly

@@ -98,3 +98,19 @@ def test_reduce_is_exact_fp32_then_one_rounding_owner_first():
     two = oc.reduce_rows([torch.cat([a, a]), torch.cat([b, b])], 0, torch.float16)
     assert two.item() == float(torch.tensor(1.0 + 2.0**-10).half())  # the sum is representable: no double rounding
     assert oc.expected_counters([256, 128], epoch=3) == [768, 384]
+
+
+def test_chained_gather_is_the_block_matrix_identity():
+    """gather_cols(shards) @ W must equal sum_p shard_p @ W[p*Ks:(p+1)*Ks] (block product):
+    a wrong column-block order or width breaks it.  Integer-valued inputs keep fp32 exact."""
+    g = torch.Generator().manual_seed(5)
+    world, M, ks, N = 3, 7, 4, 5
+    shards = [torch.randint(-3, 4, (M, ks), generator=g).half() for _ in range(world)]
+    W = torch.randint(-3, 4, (world * ks, N), generator=g).half()
+    outs = [torch.zeros(M, N, dtype=torch.float16) for _ in range(world)]
+    gathered = oc.chained_ag_gemm_rs(shards, W, outs, rank=1)
+    assert gathered.shape == (M, world * ks)
+    assert torch.equal(gathered[:, ks:2 * ks], shards[1]) and torch.equal(gathered[:, 2 * ks:], shards[2])
+    want = sum(shards[p].float() @ W[p * ks:(p + 1) * ks].float() for p in range(world))
+    for o in outs:  # every rank receives the same full product
+        assert torch.equal(o.float(), want)

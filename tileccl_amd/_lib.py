@@ -129,6 +129,11 @@ SIGNATURES = {
         C.c_int,
         [_P(GemmDesc), _P(ScatterDesc), _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],
     ),
+    "tccl_gather_cols": (C.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _P(HeapView), _P(TransportDesc), _vp]),
+    "tccl_chained_ag_gemm_rs": (
+        C.c_int,
+        [_P(GemmDesc), _vp, _i64, _i32, _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],
+    ),
     "tccl_gemm_allgather": (
         C.c_int,
         [_P(GemmDesc), _vp, _i64, _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],

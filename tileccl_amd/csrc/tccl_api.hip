@@ -753,6 +753,44 @@ int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, 
   return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
 }
 
+int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int64_t ld_shard, int32_t M,
+                     int32_t cols, int32_t elem_bytes, const tccl_heap_view* heap, const tccl_transport_desc* tr,
+                     void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  if (!gathered || !shard || M <= 0 || cols <= 0 || ld_shard < cols || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4))
+    return fail(TCCL_ERR_INVALID, "gather_cols: bad arguments");
+  if (ld_gathered < (int64_t)cols * heap->world_size)
+    return fail(TCCL_ERR_INVALID, "gather_cols: gathered rows hold %lld elements, need %lld", (long long)ld_gathered,
+                (long long)cols * heap->world_size);
+  const int v = 16 / elem_bytes;
+  if (cols % v || ld_shard % v || ld_gathered % v || !aligned16(gathered) || !aligned16(shard))
+    return fail(TCCL_ERR_UNSUPPORTED, "gather_cols: shard rows must be multiples of 16 bytes and 16-byte aligned");
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  memset(&g, 0, sizeof g);
+  g.C = (void*)shard;
+  g.M = M;
+  g.N = cols;
+  g.ldc = ld_shard;
+  g.block_m = g.block_n = 128;
+  g.group_m = 8;
+  g.tile_rows = (M + 127) / 128;
+  g.tile_cols = (cols + 127) / 128;
+  g.xcds = 1;
+  g.span = 1;
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, elem_bytes, heap, nullptr, tr);
+  c.op = tccl::kOpGatherCols;
+  c.granularity = tccl::kBulk;
+  c.directions = TCCL_DIR_PUSH | TCCL_DIR_PULL;  // the own shard is copied, the peers' are pulled
+  c.out = (char*)gathered;
+  c.ld_out_bytes = ld_gathered * elem_bytes;
+  if ((rc = set_task_units(&c, tr, false))) return rc;
+  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+}
+
 static int fill_reduce(tccl::CommArgs* c, const void* partial, int partial_dtype, void* out, int out_dtype, int64_t ld_out,
                        int M, int N, int world, int emulate_peer) {
   if (partial_dtype != TCCL_F16 && partial_dtype != TCCL_BF16 && partial_dtype != TCCL_F32)
@@ -826,6 +864,27 @@ int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, c
   c.dst_col_off = sc->dst_col_offset;
   if ((rc = set_task_units(&c, tr, false))) return rc;
   return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+}
+
+int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* d, const void* shard, int64_t ld_shard, int32_t k_shard,
+                            const tccl_heap_view* heap, const tccl_sync_desc* sync, const tccl_transport_desc* tr,
+                            int32_t variant, void* stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  if ((rc = check_heap(heap))) return rc;
+  if (k_shard <= 0 || (int64_t)k_shard * heap->world_size != d->K)
+    return fail(TCCL_ERR_INVALID, "chained: input_shard columns (%d) * world_size (%d) != W rows (%d)", k_shard,
+                heap->world_size, d->K);
+  // Stage 1: the gathered input (gemm->A) is filled from every rank's shard.
+  if ((rc = tccl_gather_cols((void*)d->A, d->lda, shard, ld_shard, d->M, k_shard, (int32_t)dtype_size(d->in_dtype), heap, tr, stream)))
+    return rc;
+  // Stages 2 and 3: the GEMM, whose whole output goes to every peer's output.
+  tccl_scatter_desc sc;
+  sc.src_col_offset = 0;
+  sc.cols = d->N;
+  sc.dst_ld = (int32_t)d->ldc;
+  sc.dst_col_offset = 0;
+  return tccl_gemm_allscatter(d, &sc, heap, sync, tr, variant, stream);
 }
 
 int tccl_gemm_allgather(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap,

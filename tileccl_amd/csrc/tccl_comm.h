@@ -9,10 +9,12 @@
 // access (global_load_dwordx4 / global_store_dwordx4), a wavefront covers 1 KiB of a row
 // per instruction, and every thread keeps several loads in flight before its stores.
 //
-// Three operations share the machinery (reference call sites in brackets):
+// Four operations share the machinery (reference call sites in brackets):
 //   all-scatter     column block of C -> every peer's C   [patterns/_helpers.py:86-199]
 //   all-gather      row block of `out` <-> peers' `out`   [primitives/collectives.py:613-663]
 //   reduce-scatter  out = cast(sum over ranks of partial) [primitives/collectives.py:730-783]
+//   gather-columns  rank p's input shard -> column block p of this rank's gathered input
+//                   [gather worker of patterns/chained_ag_gemm_rs.py:262-340]
 // and three granularities: bulk (no waiting; the second kernel of S0), per plan tile
 // (S1: tile_wait on locks[tile]) and per TileGroup (S2: tile_wait_ge on counter[group]).
 #pragma once
@@ -26,7 +28,7 @@ typedef _Float16 f16x8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3 };
+enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3, kOpGatherCols = 4 };
 enum Granularity { kBulk = 0, kPerTile = 1, kPerGroup = 2 };
 enum { kDirPush = 1, kDirPull = 2 };
 enum { kF16 = 0, kBF16 = 1, kF32 = 2 };
@@ -42,7 +44,9 @@ struct CommArgs {
   int block_m, block_n, group_m, tile_rows, tile_cols, xcds, span;
   // all-scatter placement (elements)
   int src_col_off, cols, dst_ld, dst_col_off;
-  // all-gather: gathered output of this rank; rank r's block starts at row r*M
+  // all-gather: gathered output of this rank; rank r's block starts at row r*M.
+  // gather-columns: C is this rank's input shard (M x N), out the gathered input whose
+  // column block r (N columns wide) comes from rank r's shard.
   char* out;
   int64_t ld_out_bytes;
   // reduce-scatter: C is the partial; rs_out the owner's shard
@@ -292,6 +296,20 @@ TCCL_D bool make_xfer(const CommArgs& a, bool pull, int peer, int r0, int r1, in
     x.upr = (c1 - c0) * a.esize / 16;
     return x.dst_ranks != 0;
   }
+  if (a.op == kOpGatherCols) {
+    // Column block `owner` of this rank's gathered input is rank `owner`'s shard
+    // (chained_ag_gemm_rs.py:270-337); the "push" direction is the copy of the own shard.
+    const int owner = pull ? peer : a.rank;
+    x.src_ranks = 1u << owner;
+    x.dst_ranks = 1u << a.rank;
+    x.src_pitch = a.ldc_bytes;
+    x.dst_pitch = a.ld_out_bytes;
+    x.src_off = slice_offset(a, a.C) + r0 * x.src_pitch + (int64_t)c0 * a.esize;
+    x.dst_off = slice_offset(a, a.out) + r0 * x.dst_pitch + ((int64_t)owner * a.N + c0) * a.esize;
+    x.rows = r1 - r0;
+    x.upr = (c1 - c0) * a.esize / 16;
+    return true;
+  }
   // Reduce-scatter: rows belong to owner = row / (M / world); the owner's shard is rs_out.
   const int shard = a.M / a.world;
   const int owner = r0 / shard;
@@ -397,7 +415,7 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
   Waiter wait{a, lds_word, now_ticks() + a.spin_ticks};
   const int peers = a.world - 1;
   const bool is_rs = a.op == kOpReduceScatter;
-  const bool do_pull = !is_rs && a.op == kOpAllGather && (a.directions & kDirPull) && peers > 0;
+  const bool do_pull = (a.op == kOpAllGather || a.op == kOpGatherCols) && (a.directions & kDirPull) && peers > 0;
   const bool do_push = is_rs || (a.directions & kDirPush);
   const int unit_elems = is_rs ? 8 : 16 / a.esize;
   const int units_per_task = is_rs ? a.reduce_units : a.copy_units;
