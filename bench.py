@@ -113,7 +113,9 @@ class Workload:
             pdt = torch.bfloat16 if self.in_type == "f8" else torch.float32
             odt = torch.bfloat16 if self.in_type == "f8" else torch.float16
             self.peer_cpu = seeded((M, N), 2, 1.0, pdt)
-            self.ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=pdt, out_dtype=odt, **common) for h in self.heaps]
+            # S1 / S2 keep the partial of the rows a rank owns in the accumulators (S0, two kernels, cannot)
+            self.ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=pdt, out_dtype=odt, own_rows_in_registers=True, **common)
+                        for h in self.heaps]
             self.ops[1].partial.copy_(self.peer_cpu)
             psz = self.peer_cpu.element_size()
             self.exchange_bytes = 2.0 * M * N * psz + M * N * 2  # both partials read once, every output row written once
@@ -124,9 +126,15 @@ class Workload:
         self.B.copy_(self.B_cpu)
         self.op.mark_peers_ready()
         self.flop = 2.0 * M * N * K
+        self.own_out = {}
 
     def run(self, variant):
         self.op(self.A, self.B, variant, scale_a=self.scales[0], scale_b=self.scales[1])
+
+    def after_variant(self, variant):
+        """Keep what the variant left in the first rows of rank 0's output shard (compared in spot_check)."""
+        if self.kind == "rs":
+            self.own_out[variant] = self.op.out[:256].clone().view(__import__("torch").int16)
 
     def describe(self, variant):
         M, N, K = self.M, self.N, self.K
@@ -135,7 +143,8 @@ class Workload:
                     f"2 emulated heap slices, tiles {self.block_m}x128, variant {variant.upper()}, push+pull")
         what = "e4m3 inputs, bf16 partials and output" if self.in_type == "f8" else "fp16 inputs, fp32 partials, fp16 output"
         return (f"{self.name}: GEMM -> ReduceScatter, local {M}x{K} @ {K}x{N} ({what}), resident peer partial, "
-                f"2 emulated heap slices (both owners' reductions run), tiles {self.block_m}x128, variant {variant.upper()}")
+                f"2 emulated heap slices (both owners' reductions run), tiles {self.block_m}x128, variant {variant.upper()}"
+                + ("" if variant == "s0" else ", owned rows' partial kept in registers"))
 
     def spot_check(self):
         """Parity inside the bench: moved bytes are exact / the reduction matches the oracle on a slab."""
@@ -147,11 +156,17 @@ class Workload:
         if self.kind == "ag":
             assert torch.equal(self.op.peer_out(1)[:M], self.op.out[:M]) and torch.equal(self.op.out[M:].cpu(), self.peer_cpu)
             return
-        # the first 256 rows of owner 0's shard, handed to the oracle as the owner-0 half of a 512-row problem
+        # The first 256 rows of owner 1's shard (rank 0 always stores its partial of rows it does
+        # not own), handed to the oracle as the owner-0 half of a 512-row problem, owner's addend first.
+        half = M // 2
         pad = torch.zeros(256, self.N, dtype=self.peer_cpu.dtype)
-        slabs = [torch.cat([self.op.partial[:256].cpu(), pad]), torch.cat([self.peer_cpu[:256], pad])]
+        slabs = [torch.cat([self.peer_cpu[half:half + 256], pad]), torch.cat([self.op.partial[half:half + 256].cpu(), pad])]
         want = oracle.reduce_rows(slabs, 0, self.op.out.dtype)
-        assert torch.equal(self.op.out[:256].cpu().view(torch.int16), want.view(torch.int16))
+        assert torch.equal(self.ops[1].out[:256].cpu().view(torch.int16), want.view(torch.int16))
+        # The rows rank 0 owns: the in-register variants never store that partial, so it cannot be
+        # handed to the oracle; every variant timed must have produced the same bytes.
+        outs = list(self.own_out.values())
+        assert all(torch.equal(o, outs[0]) for o in outs[1:])
 
     def gemm_only(self):
         import ctypes as C
@@ -320,6 +335,8 @@ def main() -> int:
     for variant in wanted:
         wall, mean = time_variant(w.run, variant, args.steps, args.warmup)
         w.op.check_faults()
+        if hasattr(w, "after_variant"):
+            w.after_variant(variant)
         results[variant] = {"wall_ms": wall, "event_ms_mean": mean, "tflops": w.flop / (mean * 1e-3) / 1e12,
                             "wall_tflops": w.flop / (wall * 1e-3) / 1e12}
     w.spot_check()

@@ -89,8 +89,17 @@ typedef struct tccl_gemm_desc {
   int32_t block_m, block_n, group_m; /* plan tile and swizzle band: 128/128/8 or 256/128/8 */
   int32_t num_wgs;   /* GEMM workgroups; 0 = library default for the device */
   int32_t macro_tile; /* output tile one workgroup computes: 0 = choose by shape, 128, or 256 */
-  int32_t reserved[2];
+  int32_t flags;      /* TCCL_GEMM_* bits */
+  int32_t reserved;
 } tccl_gemm_desc;
+
+/* tccl_gemm_reducescatter, variants S1 / S2 on the 256 x 256 tile with shards of whole tiles:
+ * the partial of the rows this rank owns stays in the accumulators, takes the peers' partials
+ * in the GEMM epilogue and is never stored to gemm->C (those rows of C keep their old
+ * contents); the output is bit-identical to storing and reducing.  Ignored elsewhere.
+ * (The reference's fused proof kernels have no counterpart in its tree; tile_reduce_scatter,
+ * primitives/collectives.py:730-783, always reads a stored partial.) */
+#define TCCL_GEMM_OWN_ROWS_IN_REGISTERS 1
 
 /* ---- per-launch synchronisation words ------------------------------------------------
  * Stands in for the lock tensor of WGSpecializedPattern (wg_specialized.py:104-124) and

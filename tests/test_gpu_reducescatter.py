@@ -100,6 +100,52 @@ def test_three_ranks_sum_order_owner_first(lib, variant, macro, M):
             h.cleanup()
 
 
+@pytest.mark.parametrize("variant", ["s1", "s2"])
+@pytest.mark.parametrize("world,M,partial_dtype,out_dtype", [
+    (2, 512, torch.float32, torch.float16),
+    (2, 1024, torch.bfloat16, torch.bfloat16),
+    (3, 768, torch.float32, torch.bfloat16),
+])
+def test_own_rows_kept_in_registers_give_the_same_bytes(lib, variant, world, M, partial_dtype, out_dtype):
+    """Large-tile kernel with the owned rows' partial kept in the accumulators: every output
+    equals the oracle's reduction of the stored partials of a plain run bit for bit (three
+    ranks: order-sensitive magnitudes), the owned rows of `partial` are never written, the
+    other rows are."""
+    N, K = 264, 64
+    in_dtype = torch.bfloat16 if partial_dtype == torch.bfloat16 else torch.float16
+    A_cpu, B_cpu = seeded((M, K), 0, in_dtype), seeded((K, N), 1, in_dtype, scale=1 / 8)
+    peers_cpu = {p: seeded((M, N), 10 + p, partial_dtype) * (1000.0 if world == 3 else 1.0) for p in range(1, world)}
+
+    def run(flag):
+        heaps, ops = make(world, M, N, partial_dtype=partial_dtype, out_dtype=out_dtype, macro_tile=256,
+                          tau_min_bytes=1, group_m=1, own_rows_in_registers=flag)
+        try:
+            A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+            for p in range(1, world):
+                ops[p].partial.copy_(peers_cpu[p])
+            for o in ops:
+                o.out.zero_()
+            ops[0].partial.fill_(-3.0)
+            ops[0].mark_peers_ready()
+            ops[0](A, B, variant)
+            ops[0].check_faults()
+            return ops[0].partial.cpu(), [o.out.cpu() for o in ops]
+        finally:
+            for h in heaps:
+                h.cleanup()
+
+    plain_partial, plain_outs = run(False)
+    kept_partial, kept_outs = run(True)
+    shard = M // world
+    partials = [plain_partial] + [peers_cpu[p] for p in range(1, world)]
+    for owner in range(world):
+        want = oracle.reduce_rows(partials, owner, out_dtype)
+        assert torch.equal(bits(plain_outs[owner]), bits(want)), owner
+        assert torch.equal(bits(kept_outs[owner]), bits(want)), owner
+    assert torch.all(kept_partial[:shard] == -3.0)  # never stored
+    assert torch.equal(bits(kept_partial[shard:]), bits(plain_partial[shard:]))
+
+
 def test_baseline_config_3_properties(lib):
     """8192x2048 @ 2048x4096 fp16, peer partial fp32 N(0,1): variants agree byte for byte,
     the result equals the oracle on a slab, counters match the plan."""

@@ -64,6 +64,7 @@ def gemm_desc(
     alpha: float = 1.0,
     num_wgs: int = 0,
     macro_tile: int = 0,
+    flags: int = 0,
 ) -> _lib.GemmDesc:
     if not (A.is_cuda and B.is_cuda and C_out.is_cuda):
         raise ValueError("GEMM operands must be device tensors")
@@ -84,6 +85,7 @@ def gemm_desc(
     d.block_m, d.block_n, d.group_m = int(block_m), int(block_n), int(group_m)
     d.num_wgs = int(num_wgs)
     d.macro_tile = int(macro_tile)
+    d.flags = int(flags)
     return d
 
 

@@ -55,8 +55,12 @@ class GemmDesc(C.Structure):
         ("group_m", C.c_int32),
         ("num_wgs", C.c_int32),
         ("macro_tile", C.c_int32),
-        ("reserved", C.c_int32 * 2),
+        ("flags", C.c_int32),
+        ("reserved", C.c_int32),
     ]
+
+
+GEMM_OWN_ROWS_IN_REGISTERS = 1  # TCCL_GEMM_OWN_ROWS_IN_REGISTERS
 
 
 class SyncDesc(C.Structure):

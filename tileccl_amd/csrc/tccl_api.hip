@@ -432,7 +432,7 @@ bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
 }
 
 // A reduce-scatter whose reduction the large-tile kernel can perform tile by tile.
-bool build_reduce(const tccl::CommArgs& c, const tccl_sync_desc* sync, tccl::ReduceArgs* r, tccl::Macro* m) {
+bool build_reduce(const tccl::CommArgs& c, const tccl_sync_desc* sync, int flags, tccl::ReduceArgs* r, tccl::Macro* m) {
   memset(r, 0, sizeof *r);
   if (c.op != tccl::kOpReduceScatter || c.world <= 1 || c.M % c.world) return false;
   const int shard = c.M / c.world;
@@ -445,6 +445,7 @@ bool build_reduce(const tccl::CommArgs& c, const tccl_sync_desc* sync, tccl::Red
   r->emulate_peer = c.emulate_peer;
   r->shard_rows = shard;
   r->out_bf16 = c.out_dtype == tccl::kBF16;
+  r->own_in_registers = (flags & TCCL_GEMM_OWN_ROWS_IN_REGISTERS) != 0;
   r->heap_bases = c.heap_bases;
   r->out = c.rs_out;
   r->ld_out = c.ld_rs_out_bytes / 2;
@@ -530,7 +531,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     // pulls (and, for a reduce-scatter, the reductions).
     if (build_push(c, g, &f.push)) c.directions &= ~tccl::kDirPush;
     memset(&f.reduce, 0, sizeof f.reduce);
-    if (build_reduce(c, sync, &f.reduce, &f.m)) {
+    if (build_reduce(c, sync, d->flags, &f.reduce, &f.m)) {
       c.op = tccl::kOpNone;
       memset(&f.pull, 0, sizeof f.pull);
     } else if (build_background(c, &f.pull)) {

@@ -97,6 +97,7 @@ struct ReduceArgs {
   int rank, world, emulate_peer;
   int shard_rows;                 // rows per owner; a multiple of the 256-row tile
   int out_bf16;                   // output element: 0 fp16, 1 bf16
+  int own_in_registers;           // own rows: sum the peers' partials onto the accumulators, store no partial
   const int64_t* heap_bases;
   const char* out;                // the output shard in this rank's slice (the partial is the GEMM's C)
   int64_t ld_out;                 // output pitch in elements
@@ -198,6 +199,11 @@ struct Gemm256 {
   char* lds1;  // stage 1
   char* bg;    // landing slots of the background transfer
   const int tid, lane, wave, wm, wn;
+  // A per-lane value the optimiser must treat as new at this point (blocks hoisting of what is derived from it).
+  static TCCL_D int fresh(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+  }
 
   TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, int reduce_args_offset, char* stage0,
                  char* stage1, char* landing)
@@ -710,7 +716,11 @@ struct Gemm256 {
     constexpr int kChunks = kRowBytes / 16;
     constexpr int kPerChunk = 16 / kEsz;
     char* win = lds + wave * (32 * 64 * 4);  // 8 KiB per wave, 64 KiB in all: inside stage 0
-    const int half = lane >> 5, l32 = lane & 31;
+    // The lane id is taken afresh: derived from the member, every store offset below is
+    // invariant across tiles, gets hoisted out of the tile loop and occupies registers all
+    // through the K loop.
+    const int ln = fresh(lane);
+    const int half = ln >> 5, l32 = ln & 31;
     OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
     const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
     // Fields are read through the argument block itself: a local copy would sit in scalar
@@ -748,7 +758,7 @@ struct Gemm256 {
       bool live[kRounds];
 #pragma unroll
       for (int r = 0; r < kRounds; ++r) {
-        const int idx = lane + 64 * r;
+        const int idx = ln + 64 * r;
         const int row = idx / kChunks, chunk = idx % kChunks;
         v[r] = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
         lrow[r] = wm * 128 + bi * 32 + row;
@@ -770,6 +780,114 @@ struct Gemm256 {
             __builtin_amdgcn_raw_buffer_store_b128(v[r], rt, (uint32_t)((lrow[r] * push_ld + lcol[r]) * kEsz), 0, kCoherent);
         }
       }
+    }
+  }
+
+  typedef const __attribute__((address_space(4))) ReduceArgs* ReducePtr;
+
+  // Epilogue of a tile whose rows this rank owns, reduce-scatter with the partial kept in
+  // registers: each 32-row slab is rounded to the partial type and staged through LDS exactly
+  // as epilogue() does, but instead of being stored it takes the peers' partials of the same
+  // 16-byte chunks (ascending rank: the owner's addend, this one, comes first) in fp32, is
+  // rounded once to the output type and lands in the output shard.  The bytes equal those of
+  // storing the partial and reducing it afterwards; 64 MiB less is written and read at c3.
+  TCCL_D void epilogue_reduce(ReducePtr ra, int row0, int col0, const f32x16 (&acc)[4][2]) const {
+    constexpr int kEsz = sizeof(OutT);
+    constexpr int kRowBytes = 64 * kEsz;
+    constexpr int kChunks = kRowBytes / 16;
+    constexpr int kPerChunk = 16 / kEsz;
+    constexpr int kRounds = (32 * kChunks) / 64;
+    char* win = lds + wave * (32 * 64 * 4);
+    const int ln = fresh(lane);  // as in epilogue(): keeps the offsets below out of the K loop's registers
+    const int half = ln >> 5, l32 = ln & 31;
+    const int world = ra->world, rank = ra->rank;
+    const int64_t my_base = ra->heap_bases[rank];
+    const int64_t tile_off = ((int64_t)row0 * g.ldc + col0) * kEsz;
+    const uint32_t ld_out = (uint32_t)ra->ld_out;
+    const __amdgpu_buffer_rsrc_t r_out =
+        window((int64_t)(uintptr_t)ra->out + ((int64_t)(row0 - rank * ra->shard_rows) * ra->ld_out + col0) * 2);
+    const bool bf = ra->out_bf16 != 0;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi) {
+      __syncthreads();
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n_local = bj * 32 + 8 * q + 4 * half;
+          OutT v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[bi][bj][4 * q + e] * g.alpha);
+          const int byte = n_local * kEsz;
+          const int chunk = (byte >> 4) ^ (l32 & 7);
+          char* p = win + l32 * kRowBytes + chunk * 16 + (byte & 15);
+          if constexpr (kEsz == 2) {
+            uint2 u;
+            __builtin_memcpy(&u, v, 8);
+            *(uint2*)p = u;
+          } else {
+            u32x4 u;
+            __builtin_memcpy(&u, v, 16);
+            *(u32x4*)p = u;
+          }
+        }
+      __syncthreads();
+      // kBatch chunks per lane at a time: the accumulators of the later slabs are still live.
+      constexpr int kBatch = kRounds > 4 ? 4 : kRounds;
+#pragma unroll
+      for (int r0 = 0; r0 < kRounds; r0 += kBatch) {
+        uint32_t src[kBatch], dst[kBatch];
+        bool live[kBatch];
+        float sum[kBatch][8];
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+          const int idx = ln + 64 * (r0 + r);
+          const int row = idx / kChunks, chunk = idx % kChunks;
+          const u32x4 v = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
+          const int lrow = wm * 128 + bi * 32 + row, lcol = wn * 64 + chunk * kPerChunk;
+          live[r] = row0 + lrow < g.M && col0 + lcol < g.N;
+          // idle lanes re-read the tile's first chunk and store nothing
+          src[r] = live[r] ? (uint32_t)((lrow * g.ldc + lcol) * kEsz) : 0u;
+          dst[r] = (uint32_t)((lrow * ld_out + lcol) * 2);
+          int n;
+          unpack(v, sum[r], n);
+        }
+        for (int p = 0; p < world; ++p) {
+          if (p == rank) continue;
+          const __amdgpu_buffer_rsrc_t r_peer = window((int64_t)(uintptr_t)g.C + (ra->heap_bases[p] - my_base) + tile_off);
+          u32x4 addend[kBatch];
+#pragma unroll
+          for (int r = 0; r < kBatch; ++r) addend[r] = ld16<kCoherent>(r_peer, src[r]);
+#pragma unroll
+          for (int r = 0; r < kBatch; ++r) {
+            float f[8];
+            int n;
+            unpack(addend[r], f, n);
+#pragma unroll
+            for (int e = 0; e < kPerChunk; ++e) sum[r][e] += f[e];
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+          if constexpr (kPerChunk == 4) {
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            u32x2 o;
+            if (bf) {
+              const __bf16 h[4] = {(__bf16)sum[r][0], (__bf16)sum[r][1], (__bf16)sum[r][2], (__bf16)sum[r][3]};
+              __builtin_memcpy(&o, h, 8);
+            } else {
+              const _Float16 h[4] = {(_Float16)sum[r][0], (_Float16)sum[r][1], (_Float16)sum[r][2], (_Float16)sum[r][3]};
+              __builtin_memcpy(&o, h, 8);
+            }
+            if (live[r]) __builtin_amdgcn_raw_buffer_store_b64(o, r_out, dst[r], 0, kStreaming);
+          } else {
+            const u32x4 o = bf ? pack8<__bf16>(sum[r]) : pack8<_Float16>(sum[r]);
+            if (live[r]) st16<kStreaming>(r_out, dst[r], o);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one slab's addends at a time: the accumulators are still live
     }
   }
 
@@ -810,6 +928,19 @@ struct Gemm256 {
         k_step16(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
     }
+    if constexpr (kWithReduce) {
+      // Rows this rank owns, partial kept in registers: the peers' partials are added in the
+      // epilogue and the tile's partial is never stored (it is still published: the counters
+      // keep one meaning).  If the wait for the peers expires the partial is stored as usual.
+      const ReducePtr ra = late_kernarg_ptr<ReduceArgs>(reduce_offset);
+      if (ra->active && ra->own_in_registers && row0 / ra->shard_rows == ra->rank && reduce_wait(ra, s, mm, mn)) {
+        epilogue_reduce(ra, row0, col0, acc);
+        wait_vmem();
+        __syncthreads();
+        if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+        return;
+      }
+    }
     epilogue<kPolicy>(row0, col0, acc);
     if constexpr (kPolicy != 0) {
       wait_vmem();  // the tile's write-through stores have landed
@@ -824,8 +955,6 @@ struct Gemm256 {
       }
     }
   }
-
-  typedef const __attribute__((address_space(4))) ReduceArgs* ReducePtr;
 
   // Are the peers' partials of the plan tiles under macro tile (mm, mn) published?  One lane
   // waits (bounded); the verdict travels through an LDS word of the idle stage.
@@ -882,7 +1011,7 @@ struct Gemm256 {
     const __amdgpu_buffer_rsrc_t r_out = window((int64_t)(uintptr_t)ra->out + (ra->heap_bases[owner] - my_base) +
                                                 ((int64_t)(row0 - owner * ra->shard_rows) * ld_out + col0) * 2);
     const bool bf = ra->out_bf16 != 0;
-    for (int u0 = tid; u0 < total; u0 += kThreads256 * kUnroll) {
+    for (int u0 = fresh(tid); u0 < total; u0 += kThreads256 * kUnroll) {
       u32x4 mine[kUnroll];
       uint32_t src[kUnroll], dst[kUnroll];
       bool live[kUnroll];

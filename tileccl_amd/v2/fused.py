@@ -200,16 +200,23 @@ class FusedGemmReduceScatter(_FusedBase):
     ``tile_reduce_scatter``, reference primitives/collectives.py:730-783), accumulating in
     fp32.  With ``emulate_peer`` the launch also performs the other owners' reductions into
     their slices, i.e. the whole two-rank operation on one GPU.
+
+    ``own_rows_in_registers``: in the one-launch variants on the 256 x 256 tile (shards of
+    whole tiles) the rows this rank owns never leave the accumulators as a partial: the peers'
+    partials are added in the GEMM epilogue.  ``out`` is bit-identical; those rows of
+    ``partial`` keep whatever they held.  Ignored where it does not apply.
     """
 
     kind = "reduce_scatter"
 
     def __init__(self, heap: SymmetricHeap, M: int, N: int, *, partial_dtype: torch.dtype = torch.float32,
-                 out_dtype: torch.dtype = torch.float16, emulate_peer: bool = True, **kwargs) -> None:
+                 out_dtype: torch.dtype = torch.float16, emulate_peer: bool = True,
+                 own_rows_in_registers: bool = False, **kwargs) -> None:
         kwargs.setdefault("transport", build_p2p_transport_plan(comm_mode="pull", copy_elems=16384, reduce_elems=16384))
         super().__init__(heap, **kwargs)
         self.M, self.N = M, N
         self.emulate_peer = emulate_peer
+        self.own_rows_in_registers = own_rows_in_registers
         spec = reduce_scatter_spec(world_size=self.world_size)
         self.shard_rows = spec.shard_rows(M)
         self.partial = heap.allocate_tensor((M, N), partial_dtype)
@@ -228,6 +235,7 @@ class FusedGemmReduceScatter(_FusedBase):
         gemm = _launch.gemm_desc(
             A, B, self.partial, block_m=self.block_m, block_n=self.block_n, group_m=self.group_m,
             alpha=alpha, num_wgs=self.num_gemm_wgs, macro_tile=self.macro_tile,
+            flags=_lib.GEMM_OWN_ROWS_IN_REGISTERS if self.own_rows_in_registers else 0,
         )
         view, transport, sync = self._descs(_lib.DIR_PULL, variant)
         rc = _lib.load().tccl_gemm_reducescatter(
