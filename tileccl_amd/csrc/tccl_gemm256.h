@@ -398,6 +398,7 @@ struct Gemm256 {
   // Fetch the first counters before the first tile's prologue, so that the first K step can
   // already fetch a piece.
   TCCL_D void pull_prime(PullState& st, const PullArgs& a, char* landing) const {
+    if constexpr (kWithReduce) return;  // that instantiation never pulls: its launch clears PullArgs
     if (a.mode == kBgNone || st.next_slot >= a.slots) return;
     pull_select(st, a, st.next_slot);
     pull_probe(st, a, landing);
@@ -478,6 +479,7 @@ struct Gemm256 {
 
   // Store the piece sitting in landing slot `slot`, if any.  Returns whether a store was issued.
   TCCL_D bool pull_retire(PullState& st, const PullArgs& a, const char* landing, int slot) const {
+    if constexpr (kWithReduce) return false;
     if (a.mode == kBgNone || st.pending_lp[slot] < 0) return false;
     bool valid;
     uint32_t row, col;
@@ -508,6 +510,7 @@ struct Gemm256 {
   // (its previous piece was stored at the end of the step before last).  All control flow
   // here is wavefront-uniform.
   TCCL_D void pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
+    if constexpr (kWithReduce) return;
     if (a.mode == kBgNone) return;
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
@@ -560,6 +563,7 @@ struct Gemm256 {
 
   // After the last tile: finish what is in flight, move the remaining pieces, report.
   TCCL_D void pull_finish(PullState& st, const PullArgs& a, const char* landing, int num_wgs) const {
+    if constexpr (kWithReduce) return;
     if (a.mode == kBgNone) return;
     wait_vmem();
     pull_retire(st, a, landing, 0);
