@@ -5,9 +5,10 @@
 A step is one pass of the hot path over one synthetic batch.  The default workload is the
 local GEMM ``4096x1024 @ 1024x4096`` fp16 (fp32 accumulate) whose output is gathered with
 an emulated peer into ``8192x4096`` per slice, both transfer directions running through the
-one HBM (BASELINE config 1, the reference's "8192x4096x1024" row).  The other BASELINE
+one HBM (benchmark configuration 1, the reference's "8192x4096x1024" row).  The other
 configurations can be timed with ``--workload`` (c2: the larger all-gather; c3: GEMM ->
-ReduceScatter with fp32 partials; c4: the fp8 ReduceScatter).  Inputs are resident in the
+ReduceScatter with fp32 partials; c4: the fp8 ReduceScatter; ch1: the chained
+gather -> GEMM -> scatter over column shards).  Inputs are resident in the
 symmetric heap before the timed region.  Prints ONE JSON line.
 """
 
@@ -83,7 +84,7 @@ def time_variant(run, variant, steps, warmup):
 
 
 class Workload:
-    """One BASELINE configuration: heap slices, resident inputs, the fused operation."""
+    """One benchmark configuration: heap slices, resident inputs, the fused operation."""
 
     def __init__(self, name, macro_tile):
         import torch

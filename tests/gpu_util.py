@@ -7,7 +7,7 @@ import torch
 
 
 def seeded(shape, seed: int, dtype=torch.float16, scale: float = 1.0) -> torch.Tensor:
-    """fp32 normal samples from a CPU generator, scaled, then cast (BASELINE config recipe)."""
+    """fp32 normal samples from a CPU generator, scaled, then cast (the benchmark configurations' recipe)."""
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(*shape, generator=g) * scale).to(dtype)
 

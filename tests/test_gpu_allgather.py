@@ -1,7 +1,7 @@
 """GEMM-output AllGather (Gate 1) in the S0 / S1 / S2 variants against the CPU oracle.
 
 Placement and copied bytes must be bit-exact against the GEMM output; the GEMM itself is
-held to the fp32-matmul tolerance.  Full-size BASELINE configs are covered through
+held to the fp32-matmul tolerance.  The full-size benchmark configurations are covered through
 size-independent properties (both slices end identical, idempotence, counters)."""
 
 import pytest

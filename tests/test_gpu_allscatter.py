@@ -1,7 +1,7 @@
 """tileccl.ops.gemm_allscatter on the GPU for the three patterns, against the CPU oracle.
 
 Mirrors the reference's only numeric test (tests/test_gemm_allscatter_smoke.py) and adds the
-two-rank BASELINE config 0, the sharded contracts and byte-exact placement checks."""
+two-rank benchmark configuration 0 (512x512x256), the sharded contracts and byte-exact placement checks."""
 
 import pytest
 import torch

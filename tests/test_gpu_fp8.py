@@ -1,6 +1,6 @@
 """fp8 (OCP e4m3) GEMM and GEMM -> ReduceScatter on gfx950's 32x32x64 fp8 MFMA.
 
-Inputs follow the BASELINE fp8 recipe: N(0,1) samples divided by a per-tensor fp32 scale,
+Inputs follow the fp8 recipe of benchmark configuration 4: N(0,1) samples divided by a per-tensor fp32 scale,
 clipped to +-448 and rounded to e4m3; the scales' product multiplies the accumulator.
 Products of two e4m3 values are exact in fp32, so the GPU result differs from the oracle
 (dequantise, fp32 matmul) only by fp32 summation order and the output rounding; the stated

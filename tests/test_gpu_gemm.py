@@ -32,7 +32,7 @@ SHAPES = [
     (200, 136, 72),  # ragged M, N and a K tail
     (1, 8, 8),
     (130, 8, 264),
-    (512, 512, 256),  # BASELINE config 0
+    (512, 512, 256),  # benchmark configuration 0
     (1024, 4096, 1024),
 ]
 
