@@ -173,3 +173,29 @@ def test_pattern_resolution_by_name_class_instance():
         pick(WGSpecializedPattern(fake_ctx(rank=1)))
     with pytest.raises(ValueError, match="BLOCK_K=32"):
         BulkSyncPattern(ctx, BLOCK_K=32)
+
+
+def test_auto_select_reference_tree_and_measured_policy():
+    """Each branch of the reference's decision tree (auto_select.py:128-188), by hand, at its
+    default hardware (132 units, 300 GB/s -> bw_scale 1), and the policy used on MI355X."""
+    from tileccl_amd.patterns import auto_select as sel
+    from tileccl_amd.patterns.hip_patterns import BulkSyncPattern, TileGroupPattern, WGSpecializedPattern
+
+    ref = lambda M, N, K, ws: sel.reference_choice(M, N, K, ws, 132, 300.0)  # noqa: E731
+    assert ref(128, 8192, 32768, 8) == "bulk_sync"                 # M < 256
+    assert ref(4096, 4096, 16384, 8) == "fused_sequential"          # N/ws = 512 < 1024, K > 12288
+    assert ref(4096, 8192, 8192, 8) == "producer_consumer"          # N/ws = 1024 < 2048, K > 6144
+    assert ref(4096, 32768, 8192, 8) == "wg_specialized"            # 32 x 32 tiles >= 132, K > 4096
+    assert ref(256, 16384, 16384, 2) == "wg_specialized"            # 2 x 64 = 128 tiles < 132; N > 4096, K > 8192
+    assert ref(4096, 8192, 1024, 2) == "fused_sequential"           # intensity 2K = 2048 > 256, tiles > 16
+    assert ref(256, 512, 64, 2) == "bulk_sync"                      # nothing applies
+    # doubling the link bandwidth doubles the K thresholds: the producer_consumer case falls through
+    assert sel.reference_choice(4096, 8192, 8192, 8, 132, 600.0) == "fused_sequential"
+    assert sel.auto_select("gemm_allscatter", 4096, 8192, 1024, 2) is TileGroupPattern
+    assert sel.auto_select("gemm_allscatter", 4096, 8192, 1024, 1) is BulkSyncPattern
+    assert sel.auto_select("gemm_allgather", 64, 8192, 1024, 2) is TileGroupPattern
+    assert sel.auto_select("gemm_allscatter", 4096, 32768, 8192, 8, policy="reference") is WGSpecializedPattern
+    with pytest.raises(ValueError, match="Unsupported operation 'gemm'"):
+        sel.auto_select("gemm", 1, 1, 1, 1)
+    with pytest.raises(ValueError, match="unknown policy"):
+        sel.auto_select("gemm_allscatter", 1, 1, 1, 1, policy="x")

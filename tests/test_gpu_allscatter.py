@@ -82,7 +82,7 @@ def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, inspect=None,
 
 
 @pytest.mark.parametrize("pattern", PATTERNS)
-def test_baseline_config_0(lib, pattern):
+def test_benchmark_configuration_0(lib, pattern):
     """512x256 @ 256x512 fp16, seed 0, world 2, tiles 128x128: each slice ends with the full C."""
     def inspect(plans):
         if pattern == "tile_group":
@@ -168,6 +168,36 @@ def test_sharded_and_mixed_contracts(lib):
         with pytest.raises(ValueError, match="C must live in the symmetric heap"):
             A, B = ctxs[0].as_symmetric(A_cpu.cuda()), ctxs[0].as_symmetric(B_cpu.cuda())
             ops.gemm_allscatter(A, B, torch.zeros(M, N, dtype=torch.float16, device="cuda"), ctx=ctxs[0], pattern="s0")
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()
+
+
+def test_benchmark_all_patterns_table(lib):
+    """The comparison table of the reference (patterns/auto_select.py:194-308): every pattern runs,
+    rows come sorted by mean latency, and the output still holds the product."""
+    import tileccl_amd as tileccl
+    from tileccl_amd.patterns.auto_select import benchmark_all_patterns
+
+    ctxs = tileccl.init_local(world_size=2, heap_size=128 << 20)
+    try:
+        M, K, N = 512, 128, 512
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        As = [c.as_symmetric(A_cpu.cuda()) for c in ctxs]  # every rank allocates alike: offsets must match
+        Bs = [c.as_symmetric(B_cpu.cuda()) for c in ctxs]
+        A, B = As[0], Bs[0]
+        Cs = [c.zeros(M, N, dtype=torch.float16) for c in ctxs]
+        table = benchmark_all_patterns(A, B, Cs[0], ctxs[0], warmup=1, iters=3)
+        names = [r["pattern"] for r in table["results"]]
+        assert sorted(names) == ["bulk_sync", "fused_sequential", "producer_consumer", "tile_group", "wg_specialized"]
+        assert all("error" not in r and r["iters"] == 3 for r in table["results"])
+        means = [r["mean_ms"] for r in table["results"]]
+        assert means == sorted(means) and table["best"] == names[0]
+        assert (table["M"], table["N"], table["K"], table["world_size"]) == (M, N, K, 2)
+        torch.cuda.synchronize()
+        assert_gemm_close(Cs[0], A_cpu.float() @ B_cpu.float(), tight=0.004)
+        half = N // 2  # full/full: rank 0 sends its column block [0, N/2) to the peer and nothing else
+        assert torch.equal(bits(Cs[1][:, :half]), bits(Cs[0][:, :half])) and torch.all(Cs[1][:, half:] == 0)
     finally:
         for c in ctxs:
             c.heap.cleanup()

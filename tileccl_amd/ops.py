@@ -260,13 +260,17 @@ def _resolve_gemm_allscatter_contract(
     )
 
 
-def _auto_pattern(ctx, execution: PatternExecutionSpec) -> Pattern:
-    """``pattern="auto"``: TileGroup overlap when there is a peer to talk to, else plain GEMM."""
-    return TileGroupPattern(ctx) if execution.world_size > 1 else BulkSyncPattern(ctx)
+def _auto_pattern(ctx, execution: PatternExecutionSpec, hw_info: object | None = None) -> Pattern:
+    """``pattern="auto"``: the selection engine, as in the reference (ops.py:1283-1292)."""
+    from tileccl_amd.patterns.auto_select import auto_select
+
+    return auto_select(
+        "gemm_allscatter", M=execution.M, N=execution.full_N, K=execution.K,
+        world_size=execution.world_size, hw_info=hw_info, ctx=ctx,
+    )
 
 
 def _resolve_pattern_impl(*, pattern: PatternLike, ctx, execution: PatternExecutionSpec, hw_info: object | None) -> Pattern:
-    del hw_info
     if isinstance(pattern, Pattern):
         owner = getattr(pattern, "ctx", None)
         if owner is not None:
@@ -282,7 +286,7 @@ def _resolve_pattern_impl(*, pattern: PatternLike, ctx, execution: PatternExecut
                 )
         return pattern
     if pattern is None or pattern == "auto":
-        return _auto_pattern(ctx, execution)
+        return _auto_pattern(ctx, execution, hw_info)
     if isinstance(pattern, str):
         cls = _PATTERN_ALIASES.get(pattern)
         if cls is None:
