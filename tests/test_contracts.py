@@ -199,3 +199,18 @@ def test_auto_select_reference_tree_and_measured_policy():
         sel.auto_select("gemm", 1, 1, 1, 1)
     with pytest.raises(ValueError, match="unknown policy"):
         sel.auto_select("gemm_allscatter", 1, 1, 1, 1, policy="x")
+
+
+def test_support_matrix_shape():
+    """Sections and keys of the reference's matrix (support.py:67-88) on a stand-in context."""
+    import tileccl_amd
+
+    ctx = fake_ctx()
+    ctx.backend_name, ctx.device, ctx.heap = "hip", "cuda:0", None
+    m = tileccl_amd.describe_runtime_support(ctx).to_dict()
+    assert list(m) == ["context", "runtime_surface", "ops", "contracts", "execution_paths", "collectives", "memory"]
+    assert m["context"] == {"backend": "hip", "device": "cuda:0", "rank": 0, "world_size": 2, "has_heap": False,
+                            "heap_mode": None, "transport_strategy": None}
+    assert m["ops"]["gemm_allscatter"]["state"] == "partial"  # two ranks but no heap attached
+    assert m["collectives"]["allreduce"]["state"] == "unsupported"
+    assert m["execution_paths"]["tile_group"] == {"state": "supported", "detail": "one launch, per-TileGroup counters"}

@@ -30,6 +30,14 @@ def test_signal_wait_poll_semantics(heap):
     ipc.tile_signal(w, 3)
     ipc.tile_signal(w, 3)  # signalling twice is still "1"
     assert w[3].item() == 1
+    ipc.tile_poll(w, 3)  # set: returns, flag untouched
+    assert w[3].item() == 1
+    ipc.tile_wait(w, 3)  # consumes
+    assert w[3].item() == 0
+    with pytest.raises(RuntimeError, match=r"tile_wait: locks\[3\] was not signalled within 8 probes"):
+        ipc.tile_wait(w, 3, max_spins=8)
+    with pytest.raises(RuntimeError, match="tile_poll"):
+        ipc.tile_poll(w, 3, max_spins=8)
 
 
 def test_counter_semantics(heap):

@@ -266,6 +266,13 @@ def init_local(
     return contexts
 
 
+def describe_runtime_support(ctx: "TileCCLContext | None" = None):
+    """The structured support matrix of this build (reference tileccl/__init__.py:240-244)."""
+    from tileccl_amd.support import describe_runtime_support as _describe
+
+    return _describe(ctx)
+
+
 def get_rank() -> int:
     return _get_ctx().rank
 
@@ -298,6 +305,7 @@ __all__ = [
     "get_rank",
     "get_world_size",
     "current_context",
+    "describe_runtime_support",
     "TileCCLContext",
     "SymmetricHeap",
     "patterns",

@@ -39,6 +39,8 @@ _DEVICE_NAMES = {
     "translate_ptr": "tileccl_amd.v2.ipc",
     "tile_signal": "tileccl_amd.v2.ipc",
     "tile_signal_add": "tileccl_amd.v2.ipc",
+    "tile_wait": "tileccl_amd.v2.ipc",
+    "tile_poll": "tileccl_amd.v2.ipc",
     "tile_try_wait": "tileccl_amd.v2.ipc",
     "tile_try_poll": "tileccl_amd.v2.ipc",
     "tile_wait_ge": "tileccl_amd.v2.ipc",

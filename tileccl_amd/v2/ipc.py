@@ -66,6 +66,20 @@ def tile_try_poll(locks: torch.Tensor, tile_id: int, MAX_SPINS: int = 1024) -> i
     return _try(locks, tile_id, MAX_SPINS, False)
 
 
+def tile_wait(locks: torch.Tensor, tile_id: int, *, max_spins: int = 1 << 20) -> None:
+    """Consume the flag (1 -> 0) once it is set (reference ipc.py:152-168).  The reference spins
+    without end; here no device-side wait is unbounded, so after ``max_spins`` empty probes
+    this raises instead."""
+    if not _try(locks, tile_id, max_spins, True):
+        raise RuntimeError(f"tile_wait: locks[{tile_id}] was not signalled within {max_spins} probes")
+
+
+def tile_poll(locks: torch.Tensor, tile_id: int, *, max_spins: int = 1 << 20) -> None:
+    """Wait until the flag is set without consuming it (reference ipc.py:192-209); bounded like ``tile_wait``."""
+    if not _try(locks, tile_id, max_spins, False):
+        raise RuntimeError(f"tile_poll: locks[{tile_id}] was not signalled within {max_spins} probes")
+
+
 def tile_wait_ge(signals: torch.Tensor, tile_id: int, threshold: int, *, spin_limit_ns: int = 1_000_000) -> int:
     """1 once ``signals[tile_id] >= threshold``; 0 if ``spin_limit_ns`` passes first."""
     out = _result()
