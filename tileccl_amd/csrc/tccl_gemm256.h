@@ -305,9 +305,14 @@ struct Gemm256 {
   // fp8 operands of k-block kk (64 k): A rows of slab b, B columns of block b.
   TCCL_D Vec load_a8(const char* stage, const Reader& r, int kk, int b) const {
     const int half = lane >> 5;
-    const char* p = stage + r.a_base + b * 32 * kARow256 + ((((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz) << 4);
-    const u32x4 lo = *(const u32x4*)p;
-    const u32x4 hi = *(const u32x4*)((uintptr_t)p ^ 16u);
+    // The two 16-byte chunks of a lane are neighbours under the swizzle (chunk and chunk ^ 1).
+    // Both addresses are formed by adding to `stage`: flipping a bit of the pointer itself
+    // would hide that it points into LDS, and the load would become a flat load, which
+    // waits for every outstanding global load.
+    const uint32_t chunk = ((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz;
+    const char* row = stage + r.a_base + b * 32 * kARow256;
+    const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
+    const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
     typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
     const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(Vec, both);
