@@ -631,29 +631,47 @@ struct Gemm256 {
     Vec ring[4], fbr[2][2];
   };
 
-  // One K step of the fp8 path: the MFMAs of this step run from `cur` while the next step's
-  // operands stream into `nxt`.  An fp8 operand is 8 registers: the A slabs are fetched one at
-  // a time so that the fragments in flight stay within what the 16-bit path holds.
-  // Returns whether the step ended with a background store (the youngest memory operation).
-  TCCL_D bool k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
-                      PullState& pull, int parity) const {
+  // fp8 operand registers; they live across K steps.
+  struct Frags8 {
+    Vec ring[2], fb[2][2];
+  };
+
+  // One K step of the fp8 path: eight items (k-block kk of 64, A slab bi) of two MFMAs each,
+  // read from `cur` while the next step's operands stream into `nxt` (one pair of loads per
+  // item, items 0..3).  An fp8 operand is 8 registers and an fp8 MFMA lasts twice as long as a
+  // 16-bit one, so the A operand is fetched one item ahead (two register sets); the B
+  // operands of k-block 1 are fetched at item 2.  As in the 16-bit path the step's one barrier
+  // sits inside the step, before item 7: the reads of `cur` are done, the loads into `nxt`
+  // have landed, and item 7 fetches the next step's first operands from `nxt` behind it.
+  // 4096^3 e4m3: 54 us against 62 us with the barrier at the step's end.
+  TCCL_D void k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
+                      Frags8& f, PullState& pull, int parity) const {
     pull_issue(pull, pa, bg, parity);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      Vec fb[2];
-      fb[0] = load_b8(cur, rd, kk, 0);
-      fb[1] = load_b8(cur, rd, kk, 1);
-      issue_piece(nxt, src, kt_load, 2 * kk);
-      issue_piece(nxt, src, kt_load, 2 * kk + 1);
-#pragma unroll
-      for (int bi = 0; bi < 4; ++bi) {
-        const Vec fa = load_a8(cur, rd, kk, bi);
-        acc[bi][0] = Mfma<InT>::run(fb[0], fa, acc[bi][0]);
-        acc[bi][1] = Mfma<InT>::run(fb[1], fa, acc[bi][1]);
+    for (int i = 0; i < 8; ++i) {
+      const int kk = i >> 2, bi = i & 3;
+      const int j = (i + 1) & 7;
+      if (i == 7) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
       }
+      const char* from = i + 1 < 8 ? cur : nxt;
+      f.ring[(i + 1) & 1] = load_a8(from, rd, j >> 2, j & 3);
+      if (i == 2) {
+        f.fb[1][0] = load_b8(cur, rd, 1, 0);
+        f.fb[1][1] = load_b8(cur, rd, 1, 1);
+      }
+      if (i == 7) {
+        f.fb[0][0] = load_b8(nxt, rd, 0, 0);
+        f.fb[0][1] = load_b8(nxt, rd, 0, 1);
+      }
+      if (i < 4) issue_piece(nxt, src, kt_load, i);
+      acc[bi][0] = Mfma<InT>::run(f.fb[kk][0], f.ring[i & 1], acc[bi][0]);
+      acc[bi][1] = Mfma<InT>::run(f.fb[kk][1], f.ring[i & 1], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    return pull_retire(pull, pa, bg, parity ^ 1);  // behind the MFMAs: the piece the previous step fetched
+    pull_retire(pull, pa, bg, parity ^ 1);  // the piece the previous step fetched; waited for at the next barrier
   }
 
   // One K step of the 16-bit path: sixteen items (k-block kk, A slab bi) of two MFMAs each,
@@ -699,22 +717,6 @@ struct Gemm256 {
       __builtin_amdgcn_sched_barrier(0);
     }
     pull_retire(pull, pa, bg, parity ^ 1);  // the piece the previous step fetched; waited for at the next barrier
-  }
-
-  // Close a step of the fp8 path: this wave's loads into the next stage (and its background fetch) have
-  // landed; a background store issued at the very end may stay in flight.  The barrier is the
-  // bare instruction: __syncthreads() carries a workgroup-scope release fence, which on this
-  // target waits for vmcnt(0) and would wait for that store too.  What must be ordered is
-  // ordered by hand: the loads have landed (the wait), and this wave's LDS reads of the stage
-  // about to be overwritten fed MFMAs that are already issued.  The empty asm keeps the
-  // compiler from moving LDS accesses across the barrier.
-  TCCL_D void close_step(bool stored) const {
-    if (stored)
-      asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
   }
 
   // Stores the tile and, when a push is asked for, sends it to the peers from the same LDS staging.
@@ -923,9 +925,13 @@ struct Gemm256 {
     wait_vmem();
     __syncthreads();
     if constexpr (kFp8) {
+      Frags8 f;
+      f.fb[0][0] = load_b8(lds, rd, 0, 0);
+      f.fb[0][1] = load_b8(lds, rd, 0, 1);
+      f.ring[0] = load_a8(lds, rd, 0, 0);
       for (int kt = 0; kt < ksteps; kt += 2) {
-        close_step(k_step8(lds, lds1, src, rd, kt + 1, acc, pull, 0));
-        close_step(k_step8(lds1, lds, src, rd, kt + 2, acc, pull, 1));
+        k_step8(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
+        k_step8(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
     } else {
       Frags f;
