@@ -365,6 +365,12 @@ struct Gemm256 {
     int64_t pending_dst[2];  // and the destination block's address
     int lds_off;             // this wavefront's landing slots inside the landing array
     int probe_off;           // and its counter landing words
+    // What pull_collect() read out of the landing area right behind a K step's barrier: the
+    // counter word and the piece fetched at the step's start.  Read there, they are older than
+    // every operand fetch that follows, so using them later never waits for those.
+    int32_t probe_val;
+    u32x4 piece;
+    int piece_slot;          // landing slot `piece` was read from (-1: none)
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -396,6 +402,9 @@ struct Gemm256 {
     st.backoff = 0;
     st.pending_lp[0] = st.pending_lp[1] = -1;
     st.pending_dst[0] = st.pending_dst[1] = 0;
+    st.probe_val = 0;
+    st.piece = u32x4{0, 0, 0, 0};
+    st.piece_slot = -1;
     if (a.mode != kBgNone) pull_normalise(st, a);
     return st;
   }
@@ -489,7 +498,12 @@ struct Gemm256 {
     bool valid;
     uint32_t row, col;
     pull_unit(a, st.pending_lp[slot], valid, row, col);
-    const u32x4 v = *(const u32x4*)(landing + st.lds_off + slot * 1024 + lane * 16);
+    u32x4 v;
+    if (st.piece_slot == slot)
+      v = st.piece;  // already taken out of the landing slot by pull_collect()
+    else
+      v = *(const u32x4*)(landing + st.lds_off + slot * 1024 + lane * 16);
+    st.piece_slot = -1;
     // The store must use the bases of the block the piece belongs to: pieces are retired
     // before the slot selection moves on (pull_issue), except for the one in flight when it
     // does, whose bases are kept aside.
@@ -514,13 +528,25 @@ struct Gemm256 {
   // Start of a K step: learn about readiness, fetch the next piece into landing slot `slot`
   // (its previous piece was stored at the end of the step before last).  All control flow
   // here is wavefront-uniform.
+  // Right behind a K step's barrier (this wave's loads, the background fetches among them,
+  // have landed): take the counter word and the piece fetched into `slot` at the step's start
+  // out of the landing area.
+  TCCL_D void pull_collect(PullState& st, const PullArgs& a, const char* landing, int slot) const {
+    if constexpr (kWithReduce) return;
+    if (a.mode == kBgNone) return;
+    st.probe_val = *(const int32_t*)(landing + st.probe_off);
+    if (st.pending_lp[slot] >= 0) {
+      st.piece = *(const u32x4*)(landing + st.lds_off + slot * 1024 + lane * 16);
+      st.piece_slot = slot;
+    }
+  }
   TCCL_D void pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
     if constexpr (kWithReduce) return;
     if (a.mode == kBgNone) return;
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
       st.probe_group = -1;
-      const int32_t seen = uniform(*(const int32_t*)(landing + st.probe_off));
+      const int32_t seen = uniform(st.probe_val);
       if (g == st.gidx) {
         if (seen >= st.need)
           pull_group_done(st, a);
@@ -655,6 +681,7 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        pull_collect(pull, pa, bg, parity);
       }
       const char* from = i + 1 < 8 ? cur : nxt;
       f.ring[(i + 1) & 1] = load_a8(from, rd, j >> 2, j & 3);
@@ -671,7 +698,7 @@ struct Gemm256 {
       acc[bi][1] = Mfma<InT>::run(f.fb[kk][1], f.ring[i & 1], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    pull_retire(pull, pa, bg, parity ^ 1);  // the piece the previous step fetched; waited for at the next barrier
+    pull_retire(pull, pa, bg, parity);  // the piece this step fetched, collected behind the barrier
   }
 
   // One K step of the 16-bit path: sixteen items (k-block kk, A slab bi) of two MFMAs each,
@@ -707,6 +734,7 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        pull_collect(pull, pa, bg, parity);
       }
       const char* from = i + 2 < 16 ? cur : nxt;
       if ((j & 3) == 0) load_b16(from, rd, j >> 2, f.fbr[(j >> 2) & 1]);
@@ -716,7 +744,7 @@ struct Gemm256 {
       acc[bi][1] = Mfma<InT>::run(f.fbr[kk & 1][1], f.ring[i & 3], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    pull_retire(pull, pa, bg, parity ^ 1);  // the piece the previous step fetched; waited for at the next barrier
+    pull_retire(pull, pa, bg, parity);  // the piece this step fetched, collected behind the barrier
   }
 
   // Stores the tile and, when a push is asked for, sends it to the peers from the same LDS staging.
@@ -924,6 +952,7 @@ struct Gemm256 {
     for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
     wait_vmem();
     __syncthreads();
+    pull_collect(pull, pa, bg, 0);  // the counters fetched before this tile (no piece is pending here)
     if constexpr (kFp8) {
       Frags8 f;
       f.fb[0][0] = load_b8(lds, rd, 0, 0);
