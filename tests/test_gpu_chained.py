@@ -29,6 +29,7 @@ def put(ctx, cpu):
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
 @pytest.mark.parametrize("world,M,Ks,N,dtype", [
+    (1, 256, 64, 256, torch.float16),      # one rank: the gather is a plain copy, nothing is scattered
     (2, 512, 128, 512, torch.float16),
     (3, 300, 72, 264, torch.float16),      # ragged rows, K_shard not a multiple of the K step
     (2, 4096, 512, 4096, torch.bfloat16),  # large-tile kernel
