@@ -208,7 +208,11 @@ struct GemmRole {
     constexpr int kChunks = kRowBytes / 16;    // 16-byte chunks per row (8 or 16)
     constexpr int kPerChunk = 16 / kEsz;       // elements per chunk
     char* win = lds + wave * (32 * 64 * 4);    // 8 KiB window per wave (fp32 worst case)
-    const int half = lane >> 5, l32 = lane & 31;
+    // The lane id is taken afresh: what the epilogue derives from it is invariant across tiles
+    // and would otherwise be hoisted out of the tile loop and held in registers through the K loop.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int half = ln >> 5, l32 = ln & 31;
     // Stores go through a buffer resource rooted at the sub-tile so that the cache policy
     // can be chosen: plain write-back when nobody waits for the tile, device-coherent
     // write-through when a communication workgroup will read it right after the signal.
@@ -242,7 +246,7 @@ struct GemmRole {
       __syncthreads();
 #pragma unroll
       for (int r = 0; r < (32 * kChunks) / 64; ++r) {
-        const int idx = lane + 64 * r;
+        const int idx = ln + 64 * r;
         const int row = idx / kChunks, chunk = idx % kChunks;
         const u32x4 v = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
         const int lrow = wm * 64 + bi * 32 + row, lcol = wn * 64 + chunk * kPerChunk;
