@@ -110,6 +110,10 @@ class Workload:
                 o.out.zero_()
             self.ops[1].out[M:].copy_(self.peer_cpu)
             self.exchange_bytes = 4.0 * M * N * 2  # push: read + write own block; pull: read + write the peer's
+            # The same operation with only the push emulated (what one rank of a real pair does itself:
+            # the peer's block arrives by the peer's push, without work on this side).
+            self.push_only = FusedGemmAllGather(self.heaps[0], M, N, torch.float16, directions="push", **common)
+            FusedGemmAllGather(self.heaps[1], M, N, torch.float16, directions="push", **common)  # same offsets in the peer slice
         else:
             pdt = torch.bfloat16 if self.in_type == "f8" else torch.float32
             odt = torch.bfloat16 if self.in_type == "f8" else torch.float16
@@ -341,6 +345,13 @@ def main() -> int:
         results[variant] = {"wall_ms": wall, "event_ms_mean": mean, "tflops": w.flop / (mean * 1e-3) / 1e12,
                             "wall_tflops": w.flop / (wall * 1e-3) / 1e12}
     w.spot_check()
+    push_only = None
+    if getattr(w, "push_only", None) is not None:
+        w.push_only.mark_peers_ready()
+        _, mean = time_variant(lambda v: w.push_only(w.A, w.B, v), args.variant, args.steps, args.warmup)
+        w.push_only.check_faults()
+        push_only = {"variant": args.variant, "ms": round(mean, 5), "tflops": round(w.flop / (mean * 1e-3) / 1e12, 2),
+                     "note": "push direction only (32 MiB read + 32 MiB written at c1); value and roofline above emulate both directions"}
     _, gemm_mean = time_variant(w.gemm_only(), "s0", args.steps, args.warmup)  # GEMM alone, for the phase split
 
     peak = PEAK_TFLOPS[w.in_type]
@@ -380,6 +391,8 @@ def main() -> int:
             "kernel_ms": round(chosen["event_ms_mean"], 5),
         },
     }
+    if push_only is not None:
+        line["one_direction"] = push_only
     if "s0" in results and "s2" in results:
         line["s2_vs_s0_speedup"] = round(results["s0"]["event_ms_mean"] / results["s2"]["event_ms_mean"], 4)
     if "s0" in results:
