@@ -371,6 +371,16 @@ struct Gemm256 {
     int32_t probe_val;
     u32x4 piece;
     int piece_slot;          // landing slot `piece` was read from (-1: none)
+    // What the per-step code needs from PullArgs, kept in registers (reading a field through
+    // the argument block is a scalar load plus a wait that also drains the operand fetches),
+    // and piece positions that advance without divisions.
+    bool active;
+    uint32_t upr, pitch, units;
+    int pieces, slots, n_groups;
+    uint32_t adv_row, adv_col;   // what `stride` pieces add to (row, col)
+    uint32_t row, col;           // per lane: row / unit of this lane's unit of piece next_lp
+    uint32_t pend_off[2];        // per lane: byte offset of the pending piece inside its block
+    bool pend_valid[2];          // per lane: the unit exists (the last piece of a block may be short)
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -405,8 +415,42 @@ struct Gemm256 {
     st.probe_val = 0;
     st.piece = u32x4{0, 0, 0, 0};
     st.piece_slot = -1;
-    if (a.mode != kBgNone) pull_normalise(st, a);
+    st.active = a.mode != kBgNone;
+    st.upr = st.pitch = st.units = 0;
+    st.pieces = st.slots = st.n_groups = 0;
+    st.adv_row = st.adv_col = st.row = st.col = 0;
+    st.pend_off[0] = st.pend_off[1] = 0;
+    st.pend_valid[0] = st.pend_valid[1] = false;
+    if (st.active) {
+      st.upr = a.upr;
+      st.pitch = a.pitch;
+      st.units = a.units;
+      st.pieces = a.pieces;
+      st.slots = a.slots;
+      st.n_groups = a.n_groups;
+      const uint32_t adv = (uint32_t)st.stride * 64u;
+      st.adv_row = adv / st.upr;
+      st.adv_col = adv - st.adv_row * st.upr;
+      pull_normalise(st, a);
+      pull_locate(st);
+    }
     return st;
+  }
+
+  // (row, col) of this lane's unit of piece next_lp, by division: at the start and when a block is finished.
+  TCCL_D void pull_locate(PullState& st) const {
+    const uint32_t u = (uint32_t)st.next_lp * 64u + (uint32_t)lane;
+    st.row = u / st.upr;
+    st.col = u - st.row * st.upr;
+  }
+  // The same after next_lp += stride.
+  TCCL_D void pull_advance(PullState& st) const {
+    st.row += st.adv_row;
+    st.col += st.adv_col;
+    if (st.col >= st.upr) {
+      st.col -= st.upr;
+      ++st.row;
+    }
   }
 
   // Fetch the first counters before the first tile's prologue, so that the first K step can
@@ -420,7 +464,7 @@ struct Gemm256 {
 
   // Every lane fetches the same word; it is read back from LDS one K step later.
   TCCL_D void pull_probe(PullState& st, const PullArgs& a, char* landing) const {
-    if (st.gidx >= a.n_groups) return;
+    if (st.gidx >= st.n_groups) return;
     if (st.backoff > 0) {
       --st.backoff;
       return;
@@ -494,10 +538,7 @@ struct Gemm256 {
   // Store the piece sitting in landing slot `slot`, if any.  Returns whether a store was issued.
   TCCL_D bool pull_retire(PullState& st, const PullArgs& a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
-    if (a.mode == kBgNone || st.pending_lp[slot] < 0) return false;
-    bool valid;
-    uint32_t row, col;
-    pull_unit(a, st.pending_lp[slot], valid, row, col);
+    if (!st.active || st.pending_lp[slot] < 0) return false;
     u32x4 v;
     if (st.piece_slot == slot)
       v = st.piece;  // already taken out of the landing slot by pull_collect()
@@ -508,7 +549,7 @@ struct Gemm256 {
     // before the slot selection moves on (pull_issue), except for the one in flight when it
     // does, whose bases are kept aside.
     const int64_t dst = st.pending_dst[slot];
-    if (valid) st16<kStreaming>(window(dst), row * a.pitch + col * 16u, v);
+    if (st.pend_valid[slot]) st16<kStreaming>(window(dst), st.pend_off[slot], v);
     st.pending_lp[slot] = -1;
     return true;
   }
@@ -533,7 +574,7 @@ struct Gemm256 {
   // out of the landing area.
   TCCL_D void pull_collect(PullState& st, const PullArgs& a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return;
-    if (a.mode == kBgNone) return;
+    if (!st.active) return;
     st.probe_val = *(const int32_t*)(landing + st.probe_off);
     if (st.pending_lp[slot] >= 0) {
       st.piece = *(const u32x4*)(landing + st.lds_off + slot * 1024 + lane * 16);
@@ -542,7 +583,7 @@ struct Gemm256 {
   }
   TCCL_D void pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
     if constexpr (kWithReduce) return;
-    if (a.mode == kBgNone) return;
+    if (!st.active) return;
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
       st.probe_group = -1;
@@ -554,23 +595,29 @@ struct Gemm256 {
           st.backoff = 3;  // not there yet: fetching the counters every step only costs issue slots
       }
     }
-    if (st.next_slot >= a.slots) return;
+    if (st.next_slot >= st.slots) return;
     if (st.next_slot != st.slot) {
       pull_select(st, a, st.next_slot);
       pull_probe(st, a, landing);
       return;
     }
-    if (pull_last_unit(a, st.next_lp) < st.ready_units) {
-      bool valid;
-      uint32_t row, col;
-      pull_unit(a, st.next_lp, valid, row, col);
-      const uint32_t off = row * a.pitch + col * 16u;
+    const uint32_t last = (uint32_t)st.next_lp * 64u + 63u;
+    if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
+      const bool valid = (uint32_t)st.next_lp * 64u + (uint32_t)lane < st.units;
+      const uint32_t off = valid ? st.row * st.pitch + st.col * 16u : 0u;  // idle lanes touch the block's first unit
       __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)(landing + st.lds_off + slot * 1024), 16, off, 0, 0,
                                                kCoherent);
       st.pending_lp[slot] = st.next_lp;
       st.pending_dst[slot] = st.dst_base;
+      st.pend_off[slot] = off;
+      st.pend_valid[slot] = valid;
       st.next_lp += st.stride;
-      pull_normalise(st, a);
+      if (st.next_lp >= st.pieces) {  // block finished: rare, may divide
+        pull_normalise(st, a);
+        pull_locate(st);
+      } else {
+        pull_advance(st);
+      }
     }
     pull_probe(st, a, landing);  // look ahead: the next group's counters
   }
