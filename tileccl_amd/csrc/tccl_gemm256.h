@@ -24,8 +24,10 @@
 //                       receives 8 consecutive k of column j (four reads = the 32 k of 32x32x64).
 //
 // Pipeline: LDS holds two stages.  The loads of step kt+1 are issued, woven between the
-// MFMAs of step kt, into the stage step kt-1 has just left; `s_waitcnt vmcnt(0)` and one
-// barrier close the step, so a load has a full step of math (~2000 cycles) to land.
+// first MFMAs of step kt, into the stage step kt-1 has left.  The step's one barrier
+// (`s_waitcnt vmcnt(0) lgkmcnt(0)` + `s_barrier`) sits two items before the step's end: the
+// stage being read is finished with, the next one has landed, and the last items already fetch
+// the next step's first operands (see k_step16 / k_step8).
 //
 // The swapped-operand MFMA and the slab-wise epilogue are those of tccl_gemm.h.
 //
@@ -114,8 +116,9 @@ struct ReduceArgs {
 // A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
 // pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
 // contiguous stretch.  At the start of a K step a wavefront fetches its next piece straight
-// into one of its two LDS landing slots; at the end of the step, behind the MFMAs, it stores
-// the piece the previous step fetched.  A piece is fetched only once
+// into an LDS landing slot; behind the step's barrier (where its loads have landed) it reads
+// the piece into registers, and at the end of the step, behind the MFMAs, it stores it.  A
+// piece is fetched only once
 // the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
 // tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
 // counter fetches which are themselves left in flight for one K step.  What the K loops did
@@ -144,7 +147,7 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
 };
-constexpr int kBgPieceBytes = 8 * 2048;                 // two 1 KiB landing slots per wavefront (alternating K steps)
+constexpr int kBgPieceBytes = 8 * 2048;                 // two 1 KiB landing slots per wavefront
 constexpr int kBgBytes = kBgPieceBytes + 8 * 256;       // plus a fetched counter word (64 lanes x 4 B)
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
