@@ -68,6 +68,16 @@ def test_bad_descriptors_are_rejected_on_the_host(lib):
     h = _lib.HeapView(0x1000, 3, 2)
     assert lib.tccl_exchange_rows(0x1000, 8, 8, 8, 2, C.byref(h), None, None) == _lib.ERR_INVALID
     assert b"rank=3 out of range for world_size=2" in lib.tccl_last_error_string()
+    # gather-columns and the chained operation: host-side checks come before any device call
+    h2 = _lib.HeapView(0x1000, 0, 2)
+    assert lib.tccl_gather_cols(0x2000, 128, 0x1000, 64, 16, 64, 2, None, None, None) == _lib.ERR_INVALID
+    assert lib.tccl_gather_cols(0x2000, 100, 0x1000, 64, 16, 64, 2, C.byref(h2), None, None) == _lib.ERR_INVALID
+    assert b"gathered rows hold 100 elements, need 128" in lib.tccl_last_error_string()
+    assert lib.tccl_gather_cols(0x2000, 128, 0x1000, 64, 16, 60, 2, C.byref(h2), None, None) == _lib.ERR_UNSUPPORTED
+    d.A = 0x1000
+    d.K, d.lda = 192, 192
+    assert lib.tccl_chained_ag_gemm_rs(C.byref(d), 0x3000, 64, 64, C.byref(h2), None, None, _lib.S0_BULK, None) == _lib.ERR_INVALID
+    assert b"input_shard columns (64) * world_size (2) != W rows (192)" in lib.tccl_last_error_string()
     assert lib.tccl_heap_create(0, 2, None, None) == _lib.ERR_INVALID
     assert lib.tccl_heap_destroy(None) == 0
     assert lib.tccl_fill_i32(None, 0, 0, None) == 0
