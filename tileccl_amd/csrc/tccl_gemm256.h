@@ -1188,8 +1188,15 @@ struct Gemm256 {
   }
 
   TCCL_D void add_to_group(const SignalArgs& s, int group, int count) const {
-    const int32_t prev = tile_signal_add<true>(s.counter, group, count);
-    if (s.trace_ready_clock && prev + count == s.epoch * s.tile_counts[group]) s.trace_ready_clock[group] = now_ticks();
+    // The previous value is only needed for the trace stamp.  Without it the add is issued and
+    // forgotten: waiting for the old value costs a round trip that grows with the number of
+    // workgroups adding to the same word at the same moment (all of them, at c1).
+    if (s.trace_ready_clock) {
+      const int32_t prev = tile_signal_add<true>(s.counter, group, count);
+      if (prev + count == s.epoch * s.tile_counts[group]) s.trace_ready_clock[group] = now_ticks();
+    } else {
+      (void)tile_signal_add<true>(s.counter, group, count);
+    }
   }
 
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
