@@ -816,9 +816,13 @@ struct Gemm256 {
     // registers all through the K loop.
     const auto* push = late_kernarg_ptr<PushArgs>(push_offset < 0 ? 0 : push_offset);
     const int push_world = push_offset >= 0 ? push->world : 0;
+    // Each wavefront stages through its own 8 KiB window, and a wavefront's LDS operations
+    // execute in the order issued: inside the loop nothing has to wait for another wavefront,
+    // nor (as a __syncthreads() with its release fence would) for the previous slab's global
+    // stores to land.  One barrier up front: every wavefront has left the K loop's stages.
+    __syncthreads();
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
-      __syncthreads();
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
@@ -840,7 +844,7 @@ struct Gemm256 {
             *(u32x4*)p = u;
           }
         }
-      __syncthreads();
+      asm volatile("" ::: "memory");  // staged by this wavefront itself: LDS keeps the order
       constexpr int kRounds = (32 * kChunks) / 64;
       u32x4 v[kRounds];
       int lrow[kRounds], lcol[kRounds];
@@ -896,9 +900,13 @@ struct Gemm256 {
     const __amdgpu_buffer_rsrc_t r_out =
         window((int64_t)(uintptr_t)ra->out + ((int64_t)(row0 - rank * ra->shard_rows) * ra->ld_out + col0) * 2);
     const bool bf = ra->out_bf16 != 0;
+    // Each wavefront stages through its own 8 KiB window, and a wavefront's LDS operations
+    // execute in the order issued: inside the loop nothing has to wait for another wavefront,
+    // nor (as a __syncthreads() with its release fence would) for the previous slab's global
+    // stores to land.  One barrier up front: every wavefront has left the K loop's stages.
+    __syncthreads();
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
-      __syncthreads();
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
@@ -920,7 +928,7 @@ struct Gemm256 {
             *(u32x4*)p = u;
           }
         }
-      __syncthreads();
+      asm volatile("" ::: "memory");  // staged by this wavefront itself: LDS keeps the order
       // kBatch chunks per lane at a time: the accumulators of the later slabs are still live.
       constexpr int kBatch = kRounds > 4 ? 4 : kRounds;
 #pragma unroll
