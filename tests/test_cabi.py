@@ -65,6 +65,12 @@ def test_bad_descriptors_are_rejected_on_the_host(lib):
         _lib.check(_lib.ERR_UNSUPPORTED, "tccl_gemm")
     with pytest.raises(RuntimeError, match="HIP error in x: error code 2"):
         _lib.check(2, "x")
+    d.A = 0x1000
+    d.K, d.lda, d.ldb = 1 << 16, 1 << 16, 1 << 16  # B would span 8 GiB: 32-bit offsets cannot reach it
+    d.N = d.ldc = 1 << 16
+    assert lib.tccl_gemm(C.byref(d), None) == _lib.ERR_UNSUPPORTED
+    assert b"spans more than 4 GiB" in lib.tccl_last_error_string()
+    d.K, d.lda, d.ldb, d.N, d.ldc = 64, 64, 128, 128, 128
     h = _lib.HeapView(0x1000, 3, 2)
     assert lib.tccl_exchange_rows(0x1000, 8, 8, 8, 2, C.byref(h), None, None) == _lib.ERR_INVALID
     assert b"rank=3 out of range for world_size=2" in lib.tccl_last_error_string()

@@ -188,6 +188,15 @@ int check_gemm(const tccl_gemm_desc* d) {
   if (d->lda < d->K || d->ldb < d->N || d->ldc < d->N) return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
   if (d->lda % in_vec || d->ldb % in_vec || d->ldc % out_vec || !aligned16(d->A) || !aligned16(d->B) || !aligned16(d->C))
     return fail(TCCL_ERR_UNSUPPORTED, "gemm: A, B, C rows must start on 16-byte boundaries");
+  // The kernels address an operand with 32-bit byte offsets from a per-tile base: B from its
+  // first row down to row K-1, A and C over the 256 rows of a tile.
+  const int64_t limit = 0xffffffffll;
+  const int64_t b_span = ((int64_t)(d->K - 1) * d->ldb + d->N) * (int64_t)isz;
+  const int64_t a_span = (255 * d->lda + d->K) * (int64_t)isz;
+  const int64_t c_span = (255 * d->ldc + d->N) * (int64_t)osz;
+  if (b_span > limit || a_span > limit || c_span > limit)
+    return fail(TCCL_ERR_UNSUPPORTED, "gemm: an operand spans more than 4 GiB from a tile's base (B %lld, A %lld, C %lld bytes)",
+                (long long)b_span, (long long)a_span, (long long)c_span);
   return 0;
 }
 
