@@ -84,6 +84,9 @@ def test_bad_descriptors_are_rejected_on_the_host(lib):
     d.K, d.lda = 192, 192
     assert lib.tccl_chained_ag_gemm_rs(C.byref(d), 0x3000, 64, 64, C.byref(h2), None, None, _lib.S0_BULK, None) == _lib.ERR_INVALID
     assert b"input_shard columns (64) * world_size (2) != W rows (192)" in lib.tccl_last_error_string()
+    # a block whose rows reach beyond 32-bit offsets is refused before any launch
+    assert lib.tccl_exchange_rows(0x1000, 1 << 20, 4096, 4096, 2, C.byref(h2), None, None) == _lib.ERR_UNSUPPORTED
+    assert b"spans more than 4 GiB" in lib.tccl_last_error_string()
     assert lib.tccl_heap_create(0, 2, None, None) == _lib.ERR_INVALID
     assert lib.tccl_heap_destroy(None) == 0
     assert lib.tccl_fill_i32(None, 0, 0, None) == 0

@@ -491,7 +491,26 @@ bool build_push(const tccl::CommArgs& c, const tccl::GemmArgs& g, tccl::PushArgs
   return true;
 }
 
+// The communication code addresses a rectangle (at most all M rows of one block) with 32-bit
+// byte offsets from the rectangle's base.
+int check_rows_span(int64_t rows, int64_t pitch_bytes) {
+  if (rows * pitch_bytes > 0xffffffffll)
+    return fail(TCCL_ERR_UNSUPPORTED, "a block of %lld rows of %lld bytes spans more than 4 GiB", (long long)rows,
+                (long long)pitch_bytes);
+  return 0;
+}
+
+int check_comm_span(const tccl::CommArgs& c) {
+  int64_t pitch = c.ldc_bytes;
+  if (c.ld_out_bytes > pitch) pitch = c.ld_out_bytes;
+  if (c.ld_rs_out_bytes > pitch) pitch = c.ld_rs_out_bytes;
+  if ((int64_t)c.dst_ld * c.esize > pitch) pitch = (int64_t)c.dst_ld * c.esize;
+  return check_rows_span(c.M, pitch);
+}
+
 int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
+  const int span = check_comm_span(c);
+  if (span) return span;
   if (wgs < 1) wgs = 1;
   hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
   TCCL_HIP(hipGetLastError());
@@ -503,6 +522,8 @@ int bulk_comm_wgs(const tccl_device_info& dev) { return dev.compute_units * 4; }
 // GEMM (+ optional communication role) for one of the three operations.
 int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc* sync, const tccl_transport_desc* tr,
                 int variant, const tccl_device_info& dev, const tccl::GemmArgs& g, hipStream_t stream) {
+  const int span = c.op != tccl::kOpNone ? check_comm_span(c) : 0;
+  if (span) return span;
   const int total_tiles = g.tile_rows * g.tile_cols;
   const int compute = default_gemm_wgs(d, dev, total_tiles);
   tccl::SignalArgs s;
@@ -704,6 +725,7 @@ int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes,
   const int N = sc->src_col_offset + sc->cols;
   if ((rc = check_scatter(sc, M, N, elem_bytes, ldc, C))) return rc;
   if (heap->world_size == 1) return 0;
+  if ((rc = check_rows_span(M, (ldc > sc->dst_ld ? ldc : (int64_t)sc->dst_ld) * elem_bytes))) return rc;
   tccl_device_info dev;
   if ((rc = query_device(-1, &dev))) return rc;
   tccl::GemmArgs g;
@@ -739,6 +761,7 @@ int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, 
   const int v = 16 / elem_bytes;
   if (N % v || ld % v || !aligned16(out)) return fail(TCCL_ERR_UNSUPPORTED, "exchange_rows: rows must be multiples of 16 bytes");
   if (heap->world_size == 1) return 0;
+  if ((rc = check_rows_span(rows_per_rank, ld * elem_bytes))) return rc;
   tccl_device_info dev;
   if ((rc = query_device(-1, &dev))) return rc;
   tccl::GemmArgs g;
@@ -776,6 +799,7 @@ int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int
   const int v = 16 / elem_bytes;
   if (cols % v || ld_shard % v || ld_gathered % v || !aligned16(gathered) || !aligned16(shard))
     return fail(TCCL_ERR_UNSUPPORTED, "gather_cols: shard rows must be multiples of 16 bytes and 16-byte aligned");
+  if ((rc = check_rows_span(M, (ld_gathered > ld_shard ? ld_gathered : ld_shard) * elem_bytes))) return rc;
   tccl_device_info dev;
   if ((rc = query_device(-1, &dev))) return rc;
   tccl::GemmArgs g;
@@ -829,6 +853,7 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
   if (!partial || !out || M <= 0 || N <= 0 || ld_partial < N || ld_out < N) return fail(TCCL_ERR_INVALID, "reduce_rows: bad arguments");
   const int esize = (int)dtype_size(partial_dtype);
   if (!esize || ld_partial % (16 / esize)) return fail(TCCL_ERR_UNSUPPORTED, "reduce_rows: partial rows must be 16-byte multiples");
+  if ((rc = check_rows_span(M, ld_partial * esize)) || (rc = check_rows_span(M, ld_out * 4))) return rc;
   tccl_device_info dev;
   if ((rc = query_device(-1, &dev))) return rc;
   tccl::GemmArgs g;
