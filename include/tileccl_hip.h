@@ -207,6 +207,16 @@ int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes,
  * slice; rank r's block occupies rows [r*rows_per_rank, (r+1)*rows_per_rank). */
 int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, int32_t elem_bytes,
                        const tccl_heap_view* heap, const tccl_transport_desc* transport, void* stream);
+/* tccl_copy_block: tile_put / tile_get (primitives/communication.py:133-225) for a whole
+ * rectangle, and the copy kernels of the stand-alone collectives (_allgather_kernel,
+ * _broadcast_kernel, _scatter_kernel: primitives/collectives.py:1074-1094, 1369-1389,
+ * 1595-1621).  `src` and `dst` are addresses inside the calling rank's slice; the rectangle
+ * (rows x row_bytes, pitches in bytes) is read at `src` translated into slice `src_rank`
+ * and written at `dst` translated into every slice whose bit is set in `dst_ranks`.
+ * Rows, pitches and both addresses must be multiples of 16 bytes. */
+int tccl_copy_block(void* dst, uint32_t dst_ranks, const void* src, int32_t src_rank, int32_t rows,
+                    int64_t row_bytes, int64_t src_pitch_bytes, int64_t dst_pitch_bytes,
+                    const tccl_heap_view* heap, void* stream);
 /* tccl_gather_cols: the gather worker of ChainedAGGemmRSPattern
  * (patterns/chained_ag_gemm_rs.py:262-340).  Every rank holds an M x cols `shard` at the same
  * heap offset; column block p of this rank's `gathered` (M x world*cols, leading dim

@@ -128,6 +128,44 @@ def chained_ag_gemm_rs(shards, W, outs, rank: int, alpha: float = 1.0) -> torch.
     return gathered
 
 
+# ---- stand-alone collectives on flat tensors (one entry per rank) ---------------------------
+# tile_allgather  /root/reference/tileccl/primitives/collectives.py:613-663
+# tile_scatter    :671-727      tile_reduce_scatter :730-783      tile_broadcast :791-836
+# host restatement of the reduction in the reference itself: :2513-2546 (ascending rank order
+# in the tensor dtype; here fp32, owner first, one rounding -- see the module docstring)
+
+
+def allgather(tensors):
+    """Every rank's output: the ranks' blocks one after the other."""
+    full = torch.cat([t.reshape(-1) for t in tensors])
+    return [full.clone() for _ in tensors]
+
+
+def broadcast(tensors, root: int):
+    """Every rank's tensor after the call: the root's."""
+    return [tensors[root].clone() for _ in tensors]
+
+
+def scatter(tensor_root: torch.Tensor, world: int):
+    """Rank i's output: chunk i of the root's tensor."""
+    block = tensor_root.numel() // world
+    flat = tensor_root.reshape(-1)
+    return [flat[i * block : (i + 1) * block].clone() for i in range(world)]
+
+
+def reduce_scatter(tensors, out_dtype: torch.dtype):
+    """Rank r's output: the sum over ranks of their chunk r."""
+    world = len(tensors)
+    rows = [t.reshape(world, -1) for t in tensors]
+    return [reduce_rows(rows, r, out_dtype).reshape(-1) for r in range(world)]
+
+
+def allreduce(tensors):
+    """Every rank's tensor after all calls: the reduced chunks one after the other."""
+    full = torch.cat(reduce_scatter(tensors, tensors[0].dtype))
+    return [full.clone() for _ in tensors]
+
+
 def expected_counters(tile_counts, epoch: int = 1):
     """counter[g] after ``epoch`` launches without reset: every tile of the group signalled once each."""
     return [epoch * t for t in tile_counts]

@@ -22,7 +22,7 @@ def test_every_declared_symbol_is_exported_and_typed(lib):
     from tileccl_amd import _lib
 
     names = declared_functions()
-    assert len(names) >= 21 and "tccl_gemm_allgather" in names and "tccl_chained_ag_gemm_rs" in names
+    assert len(names) >= 22 and "tccl_copy_block" in names and "tccl_gemm_allgather" in names and "tccl_chained_ag_gemm_rs" in names
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names  # the ctypes table covers the header exactly
@@ -84,6 +84,13 @@ def test_bad_descriptors_are_rejected_on_the_host(lib):
     d.K, d.lda = 192, 192
     assert lib.tccl_chained_ag_gemm_rs(C.byref(d), 0x3000, 64, 64, C.byref(h2), None, None, _lib.S0_BULK, None) == _lib.ERR_INVALID
     assert b"input_shard columns (64) * world_size (2) != W rows (192)" in lib.tccl_last_error_string()
+    # block copy: argument checks come before any device call
+    assert lib.tccl_copy_block(0x2000, 0b11, 0x1000, 2, 1, 64, 64, 64, C.byref(h2), None) == _lib.ERR_INVALID
+    assert b"src_rank=2 out of range" in lib.tccl_last_error_string()
+    assert lib.tccl_copy_block(0x2000, 0b100, 0x1000, 0, 1, 64, 64, 64, C.byref(h2), None) == _lib.ERR_INVALID
+    assert b"names ranks beyond world_size=2" in lib.tccl_last_error_string()
+    assert lib.tccl_copy_block(0x2000, 0b11, 0x1000, 0, 1, 40, 64, 64, C.byref(h2), None) == _lib.ERR_UNSUPPORTED
+    assert lib.tccl_copy_block(0x2000, 0, 0x1000, 0, 1, 64, 64, 64, C.byref(h2), None) == 0  # nobody to write to
     # a block whose rows reach beyond 32-bit offsets is refused before any launch
     assert lib.tccl_exchange_rows(0x1000, 1 << 20, 4096, 4096, 2, C.byref(h2), None, None) == _lib.ERR_UNSUPPORTED
     assert b"spans more than 4 GiB" in lib.tccl_last_error_string()

@@ -212,5 +212,6 @@ def test_support_matrix_shape():
     assert m["context"] == {"backend": "hip", "device": "cuda:0", "rank": 0, "world_size": 2, "has_heap": False,
                             "heap_mode": None, "transport_strategy": None}
     assert m["ops"]["gemm_allscatter"]["state"] == "partial"  # two ranks but no heap attached
-    assert m["collectives"]["allreduce"]["state"] == "unsupported"
+    assert sorted(m["collectives"]) == ["allgather", "allreduce", "broadcast", "reduce_scatter", "scatter"]
+    assert m["collectives"]["allreduce"]["state"] == "partial"  # needs a heap, like the ops
     assert m["execution_paths"]["tile_group"] == {"state": "supported", "detail": "one launch, per-TileGroup counters"}

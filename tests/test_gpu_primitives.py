@@ -1,0 +1,213 @@
+"""The stand-alone collectives and block put / get on the GPU, against the CPU oracle.
+
+Ranks are emulated as slices of one arena and call one after the other, as the reference's
+single-process heaps do (primitives/collectives.py:2513-2546).  Copies are compared byte for
+byte; reductions bit for bit with the oracle (fp32 accumulate, owner first) and within one
+rounding of the reference's own restatement (ascending ranks in the tensor dtype)."""
+
+import pytest
+import torch
+
+from oracle import collectives as oracle
+from tests.gpu_util import bits, into_heap, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def heaps_of(world, size=64 << 20):
+    from tileccl_amd.memory.symmetric_heap import SymmetricHeap
+
+    return SymmetricHeap.create_all(size=size, world_size=world)
+
+
+def close(heaps):
+    for h in heaps:
+        h.cleanup()
+
+
+@pytest.mark.parametrize("world,block,dtype", [(2, 4096, torch.float16), (3, 40, torch.float32), (4, 1 << 20, torch.bfloat16),
+                                               (8, 8, torch.float16), (2, 16, torch.int8)])
+def test_allgather_every_rank_gets_the_concatenation(lib, world, block, dtype):
+    from tileccl_amd.primitives import allgather
+
+    heaps = heaps_of(world, 128 << 20)
+    try:
+        if dtype == torch.int8:
+            cpu = [torch.randint(-128, 127, (block,), dtype=torch.int8, generator=torch.Generator().manual_seed(r)) for r in range(world)]
+        else:
+            cpu = [seeded((block,), r, dtype) for r in range(world)]
+        ins = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        outs = [h.allocate_tensor((world * block,), dtype) for h in heaps]
+        for o in outs:
+            o.fill_(0)
+        # after rank 0's call alone: block 0 everywhere, the rest untouched
+        allgather(ins[0], outs[0], heaps[0])
+        torch.cuda.synchronize()
+        for o in outs:
+            assert torch.equal(o[:block].cpu(), cpu[0]) and not o[block:].any()
+        for r in range(1, world):
+            allgather(ins[r], outs[r], heaps[r])
+        torch.cuda.synchronize()
+        want = oracle.allgather(cpu)
+        for r in range(world):
+            assert torch.equal(outs[r].cpu(), want[r])
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,root", [(2, 0), (2, 1), (4, 2)])
+def test_broadcast_from_root_only(lib, world, root):
+    from tileccl_amd.primitives import broadcast
+
+    heaps = heaps_of(world)
+    try:
+        cpu = [seeded((3, 1000, 8), 10 + r) for r in range(world)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        for r in range(world):
+            if r != root:
+                broadcast(ts[r], heaps[r], root)  # a non-root call moves nothing
+        torch.cuda.synchronize()
+        for r in range(world):
+            assert torch.equal(ts[r].cpu(), cpu[r])
+        broadcast(ts[root], heaps[root], root)
+        torch.cuda.synchronize()
+        want = oracle.broadcast(cpu, root)
+        for r in range(world):
+            assert torch.equal(bits(ts[r]).cpu(), bits(want[r]))
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,root,block", [(2, 1, 2048), (3, 0, 24), (8, 5, 4096)])
+def test_scatter_chunks_to_their_ranks(lib, world, root, block):
+    from tileccl_amd.primitives import scatter
+
+    heaps = heaps_of(world)
+    try:
+        cpu = [seeded((world * block,), 20 + r, torch.bfloat16) for r in range(world)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        outs = [h.allocate_tensor((block,), torch.bfloat16) for h in heaps]
+        for o in outs:
+            o.fill_(0)
+        for r in range(world):
+            scatter(ts[r], outs[r], heaps[r], root=root)
+        torch.cuda.synchronize()
+        want = oracle.scatter(cpu[root], world)
+        for r in range(world):
+            assert torch.equal(bits(outs[r]).cpu(), bits(want[r]))
+            assert torch.equal(ts[r].cpu(), cpu[r])  # sources untouched
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,block,dtype,odtype", [
+    (2, 4096, torch.float16, torch.float16), (2, 1 << 18, torch.float32, torch.float16), (3, 72, torch.bfloat16, torch.bfloat16),
+    (4, 2048, torch.float32, torch.bfloat16), (8, 8, torch.float16, torch.float16),
+])
+def test_reduce_scatter_matches_the_oracle_bit_for_bit(lib, world, block, dtype, odtype):
+    from tileccl_amd.primitives import reduce_scatter
+
+    heaps = heaps_of(world)
+    try:
+        cpu = [seeded((world, block), 30 + r, dtype) for r in range(world)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        outs = [h.allocate_tensor((block,), odtype) for h in heaps]
+        for r in range(world):
+            reduce_scatter(ts[r], outs[r], heaps[r])
+        torch.cuda.synchronize()
+        want = oracle.reduce_scatter(cpu, odtype)
+        for r in range(world):
+            assert torch.equal(bits(outs[r]).cpu(), bits(want[r]))
+            # the reference's restatement: ascending ranks, tensor dtype (:2536-2545)
+            plain = cpu[0].reshape(world, -1)[r].clone()
+            for p in range(1, world):
+                plain = plain + cpu[p].reshape(world, -1)[r]
+            assert torch.allclose(outs[r].cpu().float(), plain.float(), rtol=2 ** -7 if odtype == torch.bfloat16 else 2 ** -9, atol=1e-2)
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,numel,dtype", [(2, 1 << 16, torch.float16), (4, 4096, torch.bfloat16), (3, 3 * 8, torch.float16)])
+def test_allreduce_in_place_any_call_order(lib, world, numel, dtype):
+    from tileccl_amd.primitives import allreduce
+
+    heaps = heaps_of(world)
+    try:
+        cpu = [seeded((numel,), 40 + r, dtype) for r in range(world)]
+        want = oracle.allreduce(cpu)
+        for order in (range(world), reversed(range(world))):
+            ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+            for r in order:
+                allreduce(ts[r], heaps[r])
+            torch.cuda.synchronize()
+            for r in range(world):
+                assert torch.equal(bits(ts[r]).cpu(), bits(want[r]))
+        # world 1: the local identity
+        solo = heaps_of(1)
+        try:
+            t = into_heap(solo[0], cpu[0])
+            allreduce(t, solo[0])
+            torch.cuda.synchronize()
+            assert torch.equal(t.cpu(), cpu[0])
+        finally:
+            close(solo)
+    finally:
+        close(heaps)
+
+
+def test_put_and_get_move_one_block(lib):
+    from tileccl_amd.primitives import copy_block, get, put
+
+    heaps = heaps_of(3)
+    try:
+        cpu = [seeded((4, 256), 50 + r) for r in range(3)]
+        a = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        b = [h.allocate_tensor((4, 256), torch.float16) for h in heaps]
+        for t in b:
+            t.fill_(0)
+        put(a[0], b[0], heaps[0], dst_rank=2)  # rank 0's a -> rank 2's b
+        torch.cuda.synchronize()
+        assert torch.equal(b[2].cpu(), cpu[0]) and not b[0].any() and not b[1].any()
+        get(b[1], a[1], heaps[1], from_rank=2)  # rank 2's a -> rank 1's b
+        torch.cuda.synchronize()
+        assert torch.equal(b[1].cpu(), cpu[2])
+        copy_block(b[0], a[0], heaps[0], src_rank=1, dst_ranks=(0, 1, 2))  # rank 1's a -> everyone's b
+        torch.cuda.synchronize()
+        for t in b:
+            assert torch.equal(t.cpu(), cpu[1])
+        for t, c in zip(a, cpu):
+            assert torch.equal(t.cpu(), c)
+    finally:
+        close(heaps)
+
+
+def test_contracts_raise_before_any_launch(lib):
+    from tileccl_amd import primitives as P
+
+    heaps = heaps_of(2)
+    try:
+        h = heaps[0]
+        t = h.allocate_tensor((64,), torch.float16)
+        o = h.allocate_tensor((128,), torch.float16)
+        with pytest.raises(ValueError, match=r"allgather output.numel must equal tensor.numel \* world_size: 64 != 64 \* 2"):
+            P.allgather(t, t, h)
+        with pytest.raises(ValueError, match=r"scatter tensor.numel must equal output.numel \* world_size: 64 != 128 \* 2"):
+            P.scatter(t, o, h)
+        with pytest.raises(ValueError, match=r"root=2 out of range \[0, 2\)"):
+            P.broadcast(t, h, root=2)
+        with pytest.raises(ValueError, match="Only op='sum' is currently supported, got 'max'"):
+            P.reduce_scatter(o, t, h, op="max")
+        with pytest.raises(ValueError, match="implementation must be one of"):
+            P.reduce_scatter(o, t, h, implementation="fast")
+        with pytest.raises(ValueError, match="output must reside in the provided SymmetricHeap for rank 0"):
+            P.allgather(t, torch.zeros(128, dtype=torch.float16, device="cuda"), h)
+        with pytest.raises(ValueError, match="allgather currently requires tensor to be contiguous"):
+            P.allgather(o.view(64, 2)[:, 0], o, h)
+        with pytest.raises(ValueError, match="not a multiple of 16 bytes"):
+            P.allgather(t[:4], t[:8], h)
+        with pytest.raises(ValueError, match="allreduce supports fp16 and bf16"):
+            P.allreduce(h.allocate_tensor((64,), torch.float32), h)
+        with pytest.raises(ValueError, match="dst_rank=5 out of range"):
+            P.put(t, t, h, dst_rank=5)
+    finally:
+        close(heaps)

@@ -114,3 +114,31 @@ def test_chained_gather_is_the_block_matrix_identity():
     want = sum(shards[p].float() @ W[p * ks:(p + 1) * ks].float() for p in range(world))
     for o in outs:  # every rank receives the same full product
         assert torch.equal(o.float(), want)
+
+
+def test_standalone_collectives_against_element_loops():
+    """allgather / broadcast / scatter / reduce_scatter / allreduce on tiny inputs, each against a
+    plain Python loop over elements and against a value a wrong index would change."""
+    world, block = 3, 8
+    # rank p, element i holds 100*p + i: every element names where it came from
+    tens = [torch.arange(world * block, dtype=torch.float32) + 100 * p for p in range(world)]
+    blocks = [t[:block].clone() for t in tens]
+    ag = oc.allgather(blocks)
+    for out in ag:
+        assert out.tolist() == [100 * (i // block) + i % block for i in range(world * block)]
+    bc = oc.broadcast(blocks, root=2)
+    assert all(t.tolist() == [200 + i for i in range(block)] for t in bc)
+    sc = oc.scatter(tens[1], world)
+    for r, out in enumerate(sc):
+        assert out.tolist() == [100 + r * block + i for i in range(block)]
+    halves = [t.half() for t in tens]
+    rs = oc.reduce_scatter(halves, torch.float16)
+    for r, out in enumerate(rs):
+        # sum over p of (100p + r*block + i) = 300 + 3*(r*block + i): exact in fp16
+        assert out.tolist() == [300 + 3 * (r * block + i) for i in range(block)]
+    ar = oc.allreduce(halves)
+    assert all(t.tolist() == [300 + 3 * i for i in range(world * block)] for t in ar)
+    # the reference's own host restatement adds the ranks in ascending order in the tensor dtype
+    # (primitives/collectives.py:2536-2545); on values exact in fp16 both orders agree
+    plain = halves[0] + halves[1] + halves[2]
+    assert torch.equal(ar[0], plain)

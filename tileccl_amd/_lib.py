@@ -133,6 +133,7 @@ SIGNATURES = {
         C.c_int,
         [_P(GemmDesc), _P(ScatterDesc), _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],
     ),
+    "tccl_copy_block": (C.c_int, [_vp, C.c_uint32, _vp, _i32, _i32, _i64, _i64, _i64, _P(HeapView), _vp]),
     "tccl_gather_cols": (C.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _P(HeapView), _P(TransportDesc), _vp]),
     "tccl_chained_ag_gemm_rs": (
         C.c_int,

@@ -786,6 +786,48 @@ int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, 
   return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
 }
 
+int tccl_copy_block(void* dst, uint32_t dst_ranks, const void* src, int32_t src_rank, int32_t rows, int64_t row_bytes,
+                    int64_t src_pitch_bytes, int64_t dst_pitch_bytes, const tccl_heap_view* heap, void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  if (!dst || !src || rows <= 0 || row_bytes <= 0 || src_pitch_bytes < row_bytes || dst_pitch_bytes < row_bytes)
+    return fail(TCCL_ERR_INVALID, "copy_block: bad arguments");
+  if (src_rank < 0 || src_rank >= heap->world_size)
+    return fail(TCCL_ERR_INVALID, "copy_block: src_rank=%d out of range for world_size=%d", src_rank, heap->world_size);
+  if (heap->world_size < 32 && (dst_ranks >> heap->world_size))
+    return fail(TCCL_ERR_INVALID, "copy_block: dst_ranks=0x%x names ranks beyond world_size=%d", dst_ranks, heap->world_size);
+  if (row_bytes % 16 || src_pitch_bytes % 16 || dst_pitch_bytes % 16 || !aligned16(dst) || !aligned16(src))
+    return fail(TCCL_ERR_UNSUPPORTED, "copy_block: rows must be multiples of 16 bytes and 16-byte aligned");
+  if (row_bytes > 0x7fffffffll) return fail(TCCL_ERR_UNSUPPORTED, "copy_block: rows of %lld bytes (limit 2 GiB)", (long long)row_bytes);
+  if ((rc = check_rows_span(rows, src_pitch_bytes > dst_pitch_bytes ? src_pitch_bytes : dst_pitch_bytes))) return rc;
+  if (dst_ranks == 0) return 0;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  memset(&g, 0, sizeof g);
+  g.C = (void*)src;
+  g.M = rows;
+  g.N = (int)row_bytes;
+  g.ldc = src_pitch_bytes;
+  g.block_m = g.block_n = 128;
+  g.group_m = 8;
+  g.tile_rows = (rows + 127) / 128;
+  g.tile_cols = (int)((row_bytes + 127) / 128);
+  g.xcds = 1;
+  g.span = 1;
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, 1, heap, nullptr, nullptr);
+  c.op = tccl::kOpCopyBlock;
+  c.granularity = tccl::kBulk;
+  c.out = (char*)dst;
+  c.ld_out_bytes = dst_pitch_bytes;
+  c.copy_src_rank = src_rank;
+  c.copy_dst_ranks = dst_ranks;
+  // 32 KiB per task, whatever the element type of the caller's data
+  c.copy_units = c.reduce_units = 2048;
+  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+}
+
 int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int64_t ld_shard, int32_t M,
                      int32_t cols, int32_t elem_bytes, const tccl_heap_view* heap, const tccl_transport_desc* tr,
                      void* stream) {

@@ -28,7 +28,7 @@ typedef _Float16 f16x8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3, kOpGatherCols = 4 };
+enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3, kOpGatherCols = 4, kOpCopyBlock = 5 };
 enum Granularity { kBulk = 0, kPerTile = 1, kPerGroup = 2 };
 enum { kDirPush = 1, kDirPull = 2 };
 enum { kF16 = 0, kBF16 = 1, kF32 = 2 };
@@ -47,8 +47,12 @@ struct CommArgs {
   // all-gather: gathered output of this rank; rank r's block starts at row r*M.
   // gather-columns: C is this rank's input shard (M x N), out the gathered input whose
   // column block r (N columns wide) comes from rank r's shard.
+  // copy-block: the rectangle at C (M rows of N bytes, esize 1) is read in slice `copy_src_rank`
+  // and written at out in every slice of the mask `copy_dst_ranks`.
   char* out;
   int64_t ld_out_bytes;
+  int copy_src_rank;
+  uint32_t copy_dst_ranks;
   // reduce-scatter: C is the partial; rs_out the owner's shard
   char* rs_out;
   int64_t ld_rs_out_bytes;
@@ -292,6 +296,19 @@ TCCL_D bool make_xfer(const CommArgs& a, bool pull, int peer, int r0, int r1, in
     x.dst_ranks = pull ? (1u << a.rank) : (all_ranks(a.world) & ~(1u << a.rank));
     x.src_off = x.dst_off = off;
     x.src_pitch = x.dst_pitch = a.ld_out_bytes;
+    x.rows = r1 - r0;
+    x.upr = (c1 - c0) * a.esize / 16;
+    return x.dst_ranks != 0;
+  }
+  if (a.op == kOpCopyBlock) {
+    // tile_put / tile_get (primitives/communication.py:133-225) on a whole rectangle: both
+    // addresses are the calling rank's own, translated into the slices named.
+    x.src_ranks = 1u << a.copy_src_rank;
+    x.dst_ranks = a.copy_dst_ranks;
+    x.src_pitch = a.ldc_bytes;
+    x.dst_pitch = a.ld_out_bytes;
+    x.src_off = slice_offset(a, a.C) + r0 * x.src_pitch + (int64_t)c0 * a.esize;
+    x.dst_off = slice_offset(a, a.out) + r0 * x.dst_pitch + (int64_t)c0 * a.esize;
     x.rows = r1 - r0;
     x.upr = (c1 - c0) * a.esize / 16;
     return x.dst_ranks != 0;

@@ -1,0 +1,24 @@
+"""Host launchers of the stand-alone collectives and of block put / get, on the HIP copy and
+reduce kernels (reference: ``/root/reference/tileccl/primitives/__init__.py``)."""
+
+from tileccl_amd.primitives.collectives import (
+    MAX_COLLECTIVE_WORLD_SIZE,
+    allgather,
+    allreduce,
+    broadcast,
+    reduce_scatter,
+    scatter,
+)
+from tileccl_amd.primitives.communication import copy_block, get, put
+
+__all__ = [
+    "MAX_COLLECTIVE_WORLD_SIZE",
+    "allgather",
+    "allreduce",
+    "broadcast",
+    "copy_block",
+    "get",
+    "put",
+    "reduce_scatter",
+    "scatter",
+]

@@ -4,8 +4,7 @@ Same shape as ``/root/reference/tileccl/support.py:29-88`` (``SupportStatus``,
 ``RuntimeSupportMatrix.to_dict()`` with its ``context / ops / contracts / execution_paths /
 collectives / memory`` sections), filled for the surface built here: the three GEMM +
 collective operations on hand-written HIP kernels, one process, ranks emulated as slices of
-one device arena.  The stand-alone collectives of the reference are not part of this build
-and are reported ``"unsupported"``.
+one device arena, plus the stand-alone collectives in their direct-write / peer-read form.
 """
 
 from __future__ import annotations
@@ -102,8 +101,13 @@ def describe_runtime_support(ctx=None) -> RuntimeSupportMatrix:
             "wg_specialized": yes("one launch, per-tile locks (also as fused_sequential / producer_consumer)"),
             "tile_group": yes("one launch, per-TileGroup counters"),
         },
-        collectives={name: no("stand-alone collective: not part of this build") for name in
-                     ("allreduce", "allgather", "broadcast", "scatter", "reduce_scatter")},
+        collectives={
+            "allreduce": SupportStatus(needs_heap, "fp16 / bf16 in place: reduce-scatter of the caller's chunk, then direct write to every rank"),
+            "allgather": SupportStatus(needs_heap, "direct write of the caller's block into every rank's output"),
+            "broadcast": SupportStatus(needs_heap, "direct write by the root"),
+            "scatter": SupportStatus(needs_heap, "direct write by the root, one chunk per rank"),
+            "reduce_scatter": SupportStatus(needs_heap, "peer reads, fp32 accumulate, fp16 / bf16 output"),
+        },
         memory={
             "symmetric_heap": yes("bump allocator over one hipMalloc arena cut into world_size slices") if has_heap
             else SupportStatus("partial", "no heap attached to this context"),
