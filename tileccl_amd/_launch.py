@@ -137,6 +137,12 @@ class SyncWords:
     ``counter[g] >= e * tile_counts[g]``, so repeated launches need no reset kernel.
     ``reset()`` zeroes the words and restarts the epoch, which is also what happens
     automatically before the 32-bit counters could overflow.
+
+    A launch recorded into a HIP graph replays with the arguments it was recorded with, so
+    its epoch cannot advance.  A TileGroup launch issued while the stream is capturing is
+    therefore preceded by fill kernels that clear the counters (recorded with it; never a
+    memset node) and runs as epoch 1; from then on every launch of these words does the
+    same, captured or not, so replays and eager launches can alternate freely.
     """
 
     locks: torch.Tensor | None = None
@@ -152,6 +158,7 @@ class SyncWords:
     epoch: int = 0
     spin_limit_ns: int = DEFAULT_SPIN_LIMIT_NS
     max_tasks_per_tile: int = 1 << 16
+    clear_every_launch: bool = False  # set by the first launch recorded into a graph
 
     def reset(self) -> None:
         for t in (self.locks, self.counter, self.barrier, self.trace_comm_counter, self.trace_start_clock,
@@ -161,6 +168,13 @@ class SyncWords:
         self.epoch = 0
 
     def next_epoch(self) -> int:
+        if self.clear_every_launch or torch.cuda.is_current_stream_capturing():
+            self.clear_every_launch = True
+            for t in (self.counter, self.barrier):
+                if t is not None:
+                    t.zero_()
+            self.epoch = 1
+            return 1
         if self.epoch >= (1 << 30) // self.max_tasks_per_tile:
             torch.cuda.current_stream().synchronize()
             self.reset()
