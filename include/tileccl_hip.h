@@ -229,7 +229,8 @@ int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int
  * shards with fp32 accumulation: out[r - row_lo] = cast(sum_p partial_p[r]) for
  * r in [row_lo, row_hi), where partial_p is `partial` translated into slice p, summed
  * local first, then peers in ascending rank.  If `emulate_peer` is non-zero the same
- * reduction is also carried out for every other rank's shard into that rank's `out`. */
+ * reduction is also carried out for every other rank's shard into that rank's `out`.
+ * `out` is fp16 or bf16, or fp32 when the partials are fp32. */
 int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_partial, void* out,
                      int32_t out_dtype, int64_t ld_out, int32_t M, int32_t N,
                      const tccl_heap_view* heap, const tccl_transport_desc* transport,

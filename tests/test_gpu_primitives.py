@@ -103,6 +103,7 @@ def test_scatter_chunks_to_their_ranks(lib, world, root, block):
 @pytest.mark.parametrize("world,block,dtype,odtype", [
     (2, 4096, torch.float16, torch.float16), (2, 1 << 18, torch.float32, torch.float16), (3, 72, torch.bfloat16, torch.bfloat16),
     (4, 2048, torch.float32, torch.bfloat16), (8, 8, torch.float16, torch.float16),
+    (2, 4096, torch.float32, torch.float32), (3, 1 << 16, torch.float32, torch.float32),
 ])
 def test_reduce_scatter_matches_the_oracle_bit_for_bit(lib, world, block, dtype, odtype):
     from tileccl_amd.primitives import reduce_scatter
@@ -122,12 +123,14 @@ def test_reduce_scatter_matches_the_oracle_bit_for_bit(lib, world, block, dtype,
             plain = cpu[0].reshape(world, -1)[r].clone()
             for p in range(1, world):
                 plain = plain + cpu[p].reshape(world, -1)[r]
-            assert torch.allclose(outs[r].cpu().float(), plain.float(), rtol=2 ** -7 if odtype == torch.bfloat16 else 2 ** -9, atol=1e-2)
+            assert torch.allclose(outs[r].cpu().float(), plain.float().to(odtype).float(),
+                                  rtol=2 ** -7 if odtype == torch.bfloat16 else 2 ** -9, atol=1e-2)
     finally:
         close(heaps)
 
 
-@pytest.mark.parametrize("world,numel,dtype", [(2, 1 << 16, torch.float16), (4, 4096, torch.bfloat16), (3, 3 * 8, torch.float16)])
+@pytest.mark.parametrize("world,numel,dtype", [(2, 1 << 16, torch.float16), (4, 4096, torch.bfloat16), (3, 3 * 8, torch.float16),
+                                               (2, 1 << 20, torch.float32)])
 def test_allreduce_in_place_any_call_order(lib, world, numel, dtype):
     from tileccl_amd.primitives import allreduce
 
@@ -205,8 +208,10 @@ def test_contracts_raise_before_any_launch(lib):
             P.allgather(o.view(64, 2)[:, 0], o, h)
         with pytest.raises(ValueError, match="not a multiple of 16 bytes"):
             P.allgather(t[:4], t[:8], h)
-        with pytest.raises(ValueError, match="allreduce supports fp16 and bf16"):
-            P.allreduce(h.allocate_tensor((64,), torch.float32), h)
+        with pytest.raises(ValueError, match="allreduce supports fp16, bf16 and fp32"):
+            P.allreduce(h.allocate_tensor((64,), torch.int32), h)
+        with pytest.raises(ValueError, match="writes fp16 or bf16"):
+            P.reduce_scatter(o, h.allocate_tensor((64,), torch.float32), h)
         with pytest.raises(ValueError, match="dst_rank=5 out of range"):
             P.put(t, t, h, dst_rank=5)
     finally:

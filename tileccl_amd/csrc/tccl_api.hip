@@ -38,7 +38,7 @@ struct DeviceCache {
   int device = -1;
   tccl_device_info info;
 };
-DeviceCache g_dev;
+thread_local DeviceCache g_dev;  // per host thread: no lock, no sharing
 
 int query_device(int device, tccl_device_info* out) {
   if (device < 0) TCCL_HIP(hipGetDevice(&device));
@@ -868,17 +868,20 @@ int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int
 }
 
 static int fill_reduce(tccl::CommArgs* c, const void* partial, int partial_dtype, void* out, int out_dtype, int64_t ld_out,
-                       int M, int N, int world, int emulate_peer) {
+                       int M, int N, int world, int emulate_peer, bool allow_f32_out = false) {
   if (partial_dtype != TCCL_F16 && partial_dtype != TCCL_BF16 && partial_dtype != TCCL_F32)
     return fail(TCCL_ERR_UNSUPPORTED, "reduce: partial dtype %d", partial_dtype);
-  if (out_dtype != TCCL_F16 && out_dtype != TCCL_BF16) return fail(TCCL_ERR_UNSUPPORTED, "reduce: output dtype must be fp16 or bf16");
+  if (out_dtype == TCCL_F32 && !(allow_f32_out && partial_dtype == TCCL_F32))
+    return fail(TCCL_ERR_UNSUPPORTED, "reduce: fp32 output only from fp32 partials in the stand-alone reduction");
+  if (out_dtype != TCCL_F16 && out_dtype != TCCL_BF16 && out_dtype != TCCL_F32)
+    return fail(TCCL_ERR_UNSUPPORTED, "reduce: output dtype must be fp16, bf16 or fp32");
   if (partial_dtype != TCCL_F32 && partial_dtype != out_dtype && !(partial_dtype == TCCL_BF16 || partial_dtype == TCCL_F16))
     return fail(TCCL_ERR_UNSUPPORTED, "reduce: dtype combination");
   if (M % world) return fail(TCCL_ERR_INVALID, "reduce: M=%d must be divisible by world_size=%d", M, world);
   if (N % 8 || ld_out % 8 || !aligned16(out) || !aligned16(partial)) return fail(TCCL_ERR_UNSUPPORTED, "reduce: rows must be multiples of 8 elements and 16-byte aligned");
   c->op = tccl::kOpReduceScatter;
   c->rs_out = (char*)out;
-  c->ld_rs_out_bytes = ld_out * 2;
+  c->ld_rs_out_bytes = ld_out * (out_dtype == TCCL_F32 ? 4 : 2);
   c->partial_dtype = partial_dtype;
   c->out_dtype = out_dtype;
   c->emulate_peer = emulate_peer;
@@ -912,7 +915,7 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
   g.span = 1;
   tccl::CommArgs c;
   fill_comm_common(&c, g, esize, heap, nullptr, tr);
-  if ((rc = fill_reduce(&c, partial, partial_dtype, out, out_dtype, ld_out, M, N, heap->world_size, emulate_peer))) return rc;
+  if ((rc = fill_reduce(&c, partial, partial_dtype, out, out_dtype, ld_out, M, N, heap->world_size, emulate_peer, true))) return rc;
   c.granularity = tccl::kBulk;
   if ((rc = set_task_units(&c, tr, true))) return rc;
   return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);

@@ -31,7 +31,7 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 enum OpKind { kOpNone = 0, kOpAllScatter = 1, kOpAllGather = 2, kOpReduceScatter = 3, kOpGatherCols = 4, kOpCopyBlock = 5 };
 enum Granularity { kBulk = 0, kPerTile = 1, kPerGroup = 2 };
 enum { kDirPush = 1, kDirPull = 2 };
-enum { kF16 = 0, kBF16 = 1, kF32 = 2 };
+enum { kF16 = 0, kBF16 = 1, kF32 = 2 };  // the codes of include/tileccl_hip.h
 
 struct CommArgs {
   int op, granularity, directions;
@@ -186,6 +186,23 @@ TCCL_D u32x4 pack8<__bf16>(const float (&f)[8]) {
 }
 
 
+// One reduced unit (8 elements) to the output: 16 bytes of fp16 / bf16, 32 bytes of fp32.
+template <typename OT, int kPolicy>
+TCCL_D void store8(__amdgpu_buffer_rsrc_t w, uint32_t off, const float (&f)[8]) {
+  if constexpr (sizeof(OT) == 4) {
+    f32x4v lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = f[e];
+      hi[e] = f[4 + e];
+    }
+    st16<kPolicy>(w, off, __builtin_bit_cast(u32x4, lo));
+    st16<kPolicy>(w, off + 16, __builtin_bit_cast(u32x4, hi));
+  } else {
+    st16<kPolicy>(w, off, pack8<OT>(f));
+  }
+}
+
 // Sum order: the owner's addend first, then the other ranks in ascending order
 // (tile_reduce_scatter: local chunk, then peers ascending; collectives.py:766-781).
 template <typename PT, typename OT, int kPolicy, int kThreads>
@@ -207,7 +224,7 @@ TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
       const int u = u0 + tid + k * kThreads;
       const uint32_t r = (uint32_t)u / (uint32_t)x.upr, c = (uint32_t)u - r * (uint32_t)x.upr;
       soff[k] = r * sp + c * kSrcUnit;
-      doff[k] = r * dp + c * 16u;
+      doff[k] = r * dp + c * (8u * (uint32_t)sizeof(OT));
       if (u >= u_hi) soff[k] = 0;  // idle lane: harmless re-read, nothing stored
       Load8<PT, kPolicy>::run(first, soff[k], acc[k]);
     }
@@ -224,7 +241,7 @@ TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
     }
 #pragma unroll
     for (int k = 0; k < kReduceUnroll; ++k)
-      if (u0 + tid + k * kThreads < u_hi) st16<kPolicy>(dst, doff[k], pack8<OT>(acc[k]));
+      if (u0 + tid + k * kThreads < u_hi) store8<OT, kPolicy>(dst, doff[k], acc[k]);
   }
 }
 
@@ -238,6 +255,9 @@ TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
     case kBF16 * 4 + kBF16: run_reduce_t<__bf16, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
     case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
     case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
+    case kF32 * 4 + kF32:  // the stand-alone reduction only: the fused launches write 16-bit shards
+      if constexpr (kPolicy == kStreaming) run_reduce_t<float, float, kPolicy, kThreads>(a, x, u_lo, u_hi);
+      break;
     default: break;
   }
 }
@@ -331,7 +351,7 @@ TCCL_D bool make_xfer(const CommArgs& a, bool pull, int peer, int r0, int r1, in
   const int shard = a.M / a.world;
   const int owner = r0 / shard;
   if (owner != a.rank && !a.emulate_peer) return false;
-  const int out_esize = 2;
+  const int out_esize = a.out_dtype == kF32 ? 4 : 2;
   x.reduce = 1;
   x.first_rank = owner;
   x.src_ranks = all_ranks(a.world);

@@ -11,7 +11,8 @@ the same movement and have no counterpart here.
 What differs, on purpose:
 
 * Reductions accumulate in fp32 (the owner's chunk first, then the other ranks ascending) and
-  round once; the reference adds in the tensor dtype.  Outputs are fp16 or bf16.
+  round once; the reference adds in the tensor dtype.  Outputs are fp16 or bf16, or fp32 for
+  fp32 tensors.
 * Blocks move in 16-byte units: a rank's block must be a multiple of 16 bytes (8 elements for
   the reductions).  The reference's one-program kernels take any power-of-two block.
 * ``allreduce`` is the reduce-scatter of the caller's chunk followed by its direct write into
@@ -145,8 +146,8 @@ def _reduce_chunk(collective: str, tensor: torch.Tensor, out: torch.Tensor, heap
     """out = sum over ranks of chunk ``heap.rank`` of their ``tensor`` (peer reads, fp32 accumulate)."""
     if tensor.dtype not in _REDUCE_IN:
         raise ValueError(f"{collective} supports fp16, bf16 and fp32 tensors, got {tensor.dtype}")
-    if out.dtype not in _REDUCE_OUT:
-        raise ValueError(f"{collective} writes fp16 or bf16, got {out.dtype}")
+    if out.dtype not in _REDUCE_OUT and not (out.dtype == torch.float32 and tensor.dtype == torch.float32):
+        raise ValueError(f"{collective} writes fp16 or bf16 (fp32 for fp32 tensors), got {out.dtype} from {tensor.dtype}")
     _whole_units(collective, block, tensor.element_size(), reduce=True)
     view = _launch.heap_view(heap.get_heap_bases(), heap.rank, heap.world_size)
     rc = _lib.load().tccl_reduce_rows(
@@ -200,8 +201,8 @@ def allreduce(tensor: torch.Tensor, heap, op: str = "sum") -> None:
     numel = int(tensor.numel())
     if world == 1 or numel == 0:
         return  # local identity (reference :2563-2583)
-    if tensor.dtype not in _REDUCE_OUT:
-        raise ValueError(f"allreduce supports fp16 and bf16 tensors, got {tensor.dtype}")
+    if tensor.dtype not in _REDUCE_IN:
+        raise ValueError(f"allreduce supports fp16, bf16 and fp32 tensors, got {tensor.dtype}")
     if numel % world:
         raise ValueError(f"allreduce tensor.numel={numel} must be divisible by world_size={world}")
     block = numel // world

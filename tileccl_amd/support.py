@@ -102,11 +102,11 @@ def describe_runtime_support(ctx=None) -> RuntimeSupportMatrix:
             "tile_group": yes("one launch, per-TileGroup counters"),
         },
         collectives={
-            "allreduce": SupportStatus(needs_heap, "fp16 / bf16 in place: reduce-scatter of the caller's chunk, then direct write to every rank"),
+            "allreduce": SupportStatus(needs_heap, "in place (fp16 / bf16 / fp32): reduce-scatter of the caller's chunk, then direct write to every rank"),
             "allgather": SupportStatus(needs_heap, "direct write of the caller's block into every rank's output"),
             "broadcast": SupportStatus(needs_heap, "direct write by the root"),
             "scatter": SupportStatus(needs_heap, "direct write by the root, one chunk per rank"),
-            "reduce_scatter": SupportStatus(needs_heap, "peer reads, fp32 accumulate, fp16 / bf16 output"),
+            "reduce_scatter": SupportStatus(needs_heap, "peer reads, fp32 accumulate; fp16 / bf16 output, fp32 from fp32 tensors"),
         },
         memory={
             "symmetric_heap": yes("bump allocator over one hipMalloc arena cut into world_size slices") if has_heap
