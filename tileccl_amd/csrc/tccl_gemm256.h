@@ -689,14 +689,17 @@ struct Gemm256 {
     if (!ok && lane == 0 && a.fault) *a.fault = 1;
     wait_vmem();
     __syncthreads();
-    // One arrival per workgroup on barrier[0]; the last one to arrive brings the other groups'
-    // words up to the same count (concurrent adds to one word cost ~7 ns each on this part).
-    if (tid == 0 && a.barrier) {
+    // Only a traced launch counts arrivals: one per workgroup on barrier[0], and the last one
+    // to arrive brings the other groups' words up to the same count and stamps the clocks.
+    // Nobody waits on these words (a pull completes on the pulling rank, whose kernel ends;
+    // pushes are announced by counter[g]), and 256 adds to one word cost ~7 ns each here,
+    // ~1 us at the very end of every launch.
+    if (tid == 0 && a.barrier && a.trace_done_clock) {
       const int32_t prev = tile_signal_add<true>(a.barrier, 0, 1);
       if (prev + 1 == a.epoch * num_wgs) {
         for (int g = 0; g < a.n_groups; ++g) {
           if (g > 0) tile_signal_add<true>(a.barrier, g, num_wgs);
-          if (a.trace_done_clock) a.trace_done_clock[g] = now_ticks();
+          a.trace_done_clock[g] = now_ticks();
         }
       }
     }
