@@ -68,19 +68,28 @@ def time_variant(run, variant, steps, warmup):
     The events are recorded on the stream the kernels are launched on (torch's current
     stream), one before the first launch and one after the last.
     """
+    import gc
+
     import torch
 
     for _ in range(warmup):
         run(variant)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    start.record()
-    for _ in range(steps):
-        run(variant)
-    stop.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # As timeit does: a full collection of the interpreter's cyclic garbage takes tens of
+    # milliseconds with torch loaded, during which nothing is enqueued and the GPU idles.
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        start.record()
+        for _ in range(steps):
+            run(variant)
+        stop.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        gc.enable()
     return wall_ms, start.elapsed_time(stop) / steps
 
 
