@@ -62,25 +62,38 @@ def quantised(shape, seed, std):
     return (x / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn), scale
 
 
+SETTLE_SECONDS = 0.05
+
+
 def time_variant(run, variant, steps, warmup):
     """(wall ms per step, HIP-event ms per launch) over exactly `steps` back-to-back launches.
 
     The events are recorded on the stream the kernels are launched on (torch's current
     stream), one before the first launch and one after the last.
+
+    Warm-up is `warmup` launches and at least SETTLE_SECONDS of them: the part lowers its clocks
+    within milliseconds of idling (the host work between two variants is enough) and takes
+    tens of milliseconds of load to raise them again (traced: the same GEMM 37 us right after
+    an idle gap, 33 us 40 ms later), so a count alone would time each variant at a different
+    point of that ramp.
     """
     import gc
 
     import torch
 
-    for _ in range(warmup):
-        run(variant)
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
     # As timeit does: a full collection of the interpreter's cyclic garbage takes tens of
     # milliseconds with torch loaded, during which nothing is enqueued and the GPU idles.
     gc.collect()
     gc.disable()
     try:
+        done, t_warm = 0, time.perf_counter()
+        while done < warmup or time.perf_counter() - t_warm < SETTLE_SECONDS:
+            for _ in range(20 if done >= warmup else warmup):
+                run(variant)
+            done += 20 if done >= warmup else warmup
+            torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         start.record()
         for _ in range(steps):
@@ -91,19 +104,6 @@ def time_variant(run, variant, steps, warmup):
     finally:
         gc.enable()
     return wall_ms, start.elapsed_time(stop) / steps
-
-
-def settle(run, seconds=0.05):
-    """Untimed launches until `seconds` have passed: the part raises its clocks over the first
-    milliseconds of load, so whichever variant is timed first would otherwise look slower
-    than the ones after it (measured: ~8 % on the first 6 ms after idle)."""
-    import torch
-
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < seconds:
-        for _ in range(20):
-            run("s0")
-        torch.cuda.synchronize()
 
 
 class Workload:
@@ -374,7 +374,6 @@ def main() -> int:
     props = get_backend().get_device_properties()
     w = (ChainedWorkload if WORKLOADS[args.workload][0] == "ch" else Workload)(args.workload, args.macro_tile)
 
-    settle(w.gemm_only())
     results = {}
     wanted = [v for v in ("s0", "s1", "s2") if v in args.variants.split(",") or v == args.variant]
     for variant in wanted:
@@ -404,6 +403,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_min_seconds": SETTLE_SECONDS,  # untimed launches continue until this much time has passed
         "ms_per_step": round(chosen["wall_ms"], 5),
         "higher_is_better": True,
         "scaling": "weak",
