@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # this script scaled by what the same counters read for the bulk copy kernel of known size
 # (profiles/fused256_kernel_<workload>_s2_counters.md).  Known only for the default tile choice.
 MEASURED_TRAFFIC_BYTES = {("c1", "s2", 0): int(176.0 * 2**20), ("c2", "s2", 0): int(351.5 * 2**20),
-                          ("c3", "s2", 0): int(520.6 * 2**20), ("c4", "s2", 0): int(607.0 * 2**20)}
+                          ("c3", "s2", 0): int(460.0 * 2**20), ("c4", "s2", 0): int(607.0 * 2**20)}
 
 WORKLOADS = {
     # name: kind, local M, N, K, block_m, input type
@@ -188,7 +188,7 @@ class Workload:
         what = "e4m3 inputs, bf16 partials and output" if self.in_type == "f8" else "fp16 inputs, fp32 partials, fp16 output"
         return (f"{self.name}: GEMM -> ReduceScatter, local {M}x{K} @ {K}x{N} ({what}), resident peer partial, "
                 f"2 emulated heap slices (both owners' reductions run), tiles {self.block_m}x128, variant {variant.upper()}"
-                + ("" if variant == "s0" else ", owned rows' partial kept in registers"))
+                + ("" if variant == "s0" else ", reductions fed from the accumulators"))
 
     def spot_check(self):
         """Parity inside the bench: moved bytes are exact / the reduction matches the oracle on a slab."""

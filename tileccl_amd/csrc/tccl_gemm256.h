@@ -887,7 +887,12 @@ struct Gemm256 {
   // 16-byte chunks (ascending rank: the owner's addend, this one, comes first) in fp32, is
   // rounded once to the output type and lands in the output shard.  The bytes equal those of
   // storing the partial and reducing it afterwards; 64 MiB less is written and read at c3.
-  TCCL_D void epilogue_reduce(ReducePtr ra, int row0, int col0, const f32x16 (&acc)[4][2]) const {
+  //
+  // `owner` is the rank whose shard the rows belong to.  For owner != rank (two ranks, the
+  // peer's reduction carried out on its behalf under single-GPU emulation) the partial is
+  // stored as well, as that peer would read it, and the sum lands in the owner's slice; with
+  // two addends the order of the sum does not matter.
+  TCCL_D void epilogue_reduce(ReducePtr ra, int row0, int col0, const f32x16 (&acc)[4][2], int owner, bool store_partial) const {
     constexpr int kEsz = sizeof(OutT);
     constexpr int kRowBytes = 64 * kEsz;
     constexpr int kChunks = kRowBytes / 16;
@@ -900,8 +905,9 @@ struct Gemm256 {
     const int64_t my_base = ra->heap_bases[rank];
     const int64_t tile_off = ((int64_t)row0 * g.ldc + col0) * kEsz;
     const uint32_t ld_out = (uint32_t)ra->ld_out;
-    const __amdgpu_buffer_rsrc_t r_out =
-        window((int64_t)(uintptr_t)ra->out + ((int64_t)(row0 - rank * ra->shard_rows) * ra->ld_out + col0) * 2);
+    const __amdgpu_buffer_rsrc_t r_out = window((int64_t)(uintptr_t)ra->out + (ra->heap_bases[owner] - my_base) +
+                                                ((int64_t)(row0 - owner * ra->shard_rows) * ra->ld_out + col0) * 2);
+    const __amdgpu_buffer_rsrc_t r_mine = window((int64_t)(uintptr_t)g.C + tile_off);
     const bool bf = ra->out_bf16 != 0;
     // Each wavefront stages through its own 8 KiB window, and a wavefront's LDS operations
     // execute in the order issued: inside the loop nothing has to wait for another wavefront,
@@ -949,6 +955,8 @@ struct Gemm256 {
           // idle lanes re-read the tile's first chunk and store nothing
           src[r] = live[r] ? (uint32_t)((lrow * g.ldc + lcol) * kEsz) : 0u;
           dst[r] = (uint32_t)((lrow * ld_out + lcol) * 2);
+          if constexpr (!kFp8)
+            if (store_partial && live[r]) __builtin_amdgcn_raw_buffer_store_b128(v, r_mine, src[r], 0, kCoherent);
           int n;
           unpack(v, sum[r], n);
         }
@@ -1038,12 +1046,20 @@ struct Gemm256 {
       // epilogue and the tile's partial is never stored (it is still published: the counters
       // keep one meaning).  If the wait for the peers expires the partial is stored as usual.
       const ReducePtr ra = late_kernarg_ptr<ReduceArgs>(reduce_offset);
-      if (ra->active && ra->own_in_registers && row0 / ra->shard_rows == ra->rank && reduce_wait(ra, s, mm, mn)) {
-        epilogue_reduce(ra, row0, col0, acc);
-        wait_vmem();
-        __syncthreads();
-        if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
-        return;
+      if (ra->active && ra->own_in_registers) {
+        const int owner = row0 / ra->shard_rows;
+        // The other owner's rows, reduced on its behalf (emulation, two ranks): the partial is
+        // stored as that owner would read it, and the same registers enter its sum.
+        // (Not in the fp8 kernels: the extra code costs them more in spilled registers than the
+        // saved read-back is worth, measured +4 % at 16384x4096x2048.)
+        const bool for_peer = !kFp8 && owner != ra->rank && ra->emulate_peer && ra->world == 2;
+        if ((owner == ra->rank || for_peer) && reduce_wait(ra, s, mm, mn)) {
+          epilogue_reduce(ra, row0, col0, acc, owner, for_peer);
+          wait_vmem();
+          __syncthreads();
+          if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+          return;
+        }
       }
     }
     epilogue<kPolicy>(row0, col0, acc);
