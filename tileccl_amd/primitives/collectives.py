@@ -25,6 +25,8 @@ Every call is asynchronous on torch's current stream.
 
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from tileccl_amd import _launch, _lib
@@ -180,10 +182,14 @@ def reduce_scatter(tensor: torch.Tensor, output: torch.Tensor, heap, op: str = "
     _reduce_chunk("reduce_scatter", tensor, output, heap, block)
 
 
+_STAGING: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()  # heap -> {(block, dtype): tensor}
+
+
 def _staging(heap, block: int, dtype: torch.dtype) -> torch.Tensor:
-    """One reduced chunk per (block, dtype), allocated from the heap on first use.  Ranks that
-    call in the same order get the same offset, like every symmetric allocation."""
-    cache = heap.__dict__.setdefault("_collective_staging", {})
+    """One reduced chunk per (block, dtype), allocated from the heap on first use (the
+    reference caches its all-reduce workspace the same way, :2792-2838).  Ranks that call in
+    the same order get the same offset, like every symmetric allocation."""
+    cache = _STAGING.setdefault(heap, {})
     key = (block, str(dtype))
     if key not in cache:
         cache[key] = heap.allocate_tensor((block,), dtype)
