@@ -1000,7 +1000,10 @@ struct Gemm256 {
   }
 
   template <int kPolicy>
-  TCCL_D void macro_tile(const SignalArgs& s, int mm, int mn, PullState& pull) const {
+  // `unpublished` carries a finished tile whose signal is still owed (-1: none): instead of
+  // waiting for its stores to land right after its epilogue, the next tile's prologue, which
+  // has to wait for its first operands anyway, publishes it.
+  TCCL_D void macro_tile(const SignalArgs& s, int mm, int mn, PullState& pull, int& unpublished) const {
     const int row0 = mm * kMacro, col0 = mn * kMacro;
     f32x16 acc[4][2];
 #pragma unroll
@@ -1019,8 +1022,9 @@ struct Gemm256 {
     __syncthreads();  // the previous tile's epilogue has left LDS
 #pragma unroll
     for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
-    wait_vmem();
+    wait_vmem();  // the first operands are there, and so is everything the previous tile stored
     __syncthreads();
+    publish_owed(s, unpublished);
     pull_collect(pull, pa, bg, 0);  // the counters fetched before this tile (no piece is pending here)
     if constexpr (kFp8) {
       Frags8 f;
@@ -1055,15 +1059,17 @@ struct Gemm256 {
         const bool for_peer = !kFp8 && owner != ra->rank && ra->emulate_peer && ra->world == 2;
         if ((owner == ra->rank || for_peer) && reduce_wait(ra, s, mm, mn)) {
           epilogue_reduce(ra, row0, col0, acc, owner, for_peer);
-          wait_vmem();
-          __syncthreads();
-          if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+          unpublished = (mm << 16) | mn;
           return;
         }
       }
     }
     epilogue<kPolicy>(row0, col0, acc);
     if constexpr (kPolicy != 0) {
+      if constexpr (!kWithReduce) {
+        unpublished = (mm << 16) | mn;
+        return;
+      }
       wait_vmem();  // the tile's write-through stores have landed
       __syncthreads();
       if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
@@ -1075,6 +1081,13 @@ struct Gemm256 {
         }
       }
     }
+  }
+
+  // Call behind a wait for this wavefront's stores and a barrier: every store of the owed tile has landed.
+  TCCL_D void publish_owed(const SignalArgs& s, int& unpublished) const {
+    if (unpublished < 0) return;
+    if (tid == 0 && s.mode != kSignalNone) publish(s, unpublished >> 16, unpublished & 0xffff);
+    unpublished = -1;
   }
 
   // Are the peers' partials of the plan tiles under macro tile (mm, mn) published?  One lane
@@ -1230,15 +1243,21 @@ struct Gemm256 {
     const int total = m.rows * m.cols;
     PullState pull = pull_begin(pa, wg, num_wgs);
     pull_prime(pull, pa, bg);
+    int unpublished = -1;
     for (int slot = wg; slot < total; slot += num_wgs) {
       const int id = tile_for_slot(slot, total, m.xcds, m.span);
       TileCoord c = macro_coords(id, m);
       c.m += m.row_shift;
       if (c.m >= m.rows) c.m -= m.rows;
       if (s.mode == kSignalNone && push_offset < 0)
-        macro_tile<0>(s, c.m, c.n, pull);
+        macro_tile<0>(s, c.m, c.n, pull, unpublished);
       else
-        macro_tile<kCoherent>(s, c.m, c.n, pull);
+        macro_tile<kCoherent>(s, c.m, c.n, pull, unpublished);
+    }
+    if (unpublished >= 0) {  // the last tile: nothing follows that would wait for its stores
+      wait_vmem();
+      __syncthreads();
+      publish_owed(s, unpublished);
     }
     pull_finish(pull, pa, bg, num_wgs);
   }
