@@ -216,3 +216,34 @@ def test_contracts_raise_before_any_launch(lib):
             P.put(t, t, h, dst_rank=5)
     finally:
         close(heaps)
+
+
+def test_copy_block_pitched_rectangle_through_the_c_abi(lib):
+    """Rows with different pitches on the two sides, a column offset, and two targets: only the
+    rectangle changes, byte for byte."""
+    import ctypes as C
+
+    from tileccl_amd import _launch, _lib
+
+    heaps = heaps_of(3)
+    try:
+        g = torch.Generator().manual_seed(7)
+        src_cpu = [torch.randint(0, 255, (64, 256), dtype=torch.uint8, generator=g) for _ in range(3)]
+        src = [into_heap(h, c) for h, c in zip(heaps, src_cpu)]
+        dst = [h.allocate_tensor((64, 512), torch.uint8) for h in heaps]
+        for t in dst:
+            t.fill_(7)
+        rows, row_bytes, r0, sc0, dc0 = 37, 160, 5, 48, 96
+        view = _launch.heap_view(heaps[1].get_heap_bases(), 1, 3)  # called by rank 1
+        rc = lib.tccl_copy_block(
+            dst[1][r0:, dc0:].data_ptr(), 0b101, src[1][r0:, sc0:].data_ptr(), 2, rows, row_bytes, 256, 512,
+            C.byref(view), _launch.stream_ptr(),
+        )
+        _lib.check(rc, "tccl_copy_block")
+        torch.cuda.synchronize()
+        want = torch.full((64, 512), 7, dtype=torch.uint8)
+        want[r0:r0 + rows, dc0:dc0 + row_bytes] = src_cpu[2][r0:r0 + rows, sc0:sc0 + row_bytes]  # read in slice 2
+        assert torch.equal(dst[0].cpu(), want) and torch.equal(dst[2].cpu(), want)
+        assert torch.all(dst[1] == 7)  # the caller's own slice was not a target
+    finally:
+        close(heaps)
