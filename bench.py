@@ -106,6 +106,25 @@ def time_variant(run, variant, steps, warmup):
     return wall_ms, start.elapsed_time(stop) / steps
 
 
+def launch_spread(run, variant, launches=100):
+    """min / median / mean of single launches, each between its own pair of HIP events, taken
+    back to back right after a timed region (so at settled clocks)."""
+    import statistics
+
+    import torch
+
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    for a, b in pairs:
+        a.record()
+        run(variant)
+        b.record()
+    torch.cuda.synchronize()
+    us = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+    return {"launches": launches, "min": round(us[0], 2), "median": round(statistics.median(us), 2),
+            "mean": round(statistics.fmean(us), 2), "max": round(us[-1], 2),
+            "note": "an event pair per launch adds 2-3 us of event handling to each interval; ms_per_step has one pair around all steps"}
+
+
 class Workload:
     """One benchmark configuration: heap slices, resident inputs, the fused operation."""
 
@@ -383,6 +402,8 @@ def main() -> int:
             w.after_variant(variant)
         results[variant] = {"wall_ms": wall, "event_ms_mean": mean, "tflops": w.flop / (mean * 1e-3) / 1e12,
                             "wall_tflops": w.flop / (wall * 1e-3) / 1e12}
+        if variant == args.variant:
+            spread = launch_spread(w.run, variant)
     w.spot_check()
     push_only = None
     if getattr(w, "push_only", None) is not None:
@@ -419,6 +440,7 @@ def main() -> int:
         "variants_ms": {v: round(r["event_ms_mean"], 5) for v, r in results.items()},
         "variants_tflops": {v: round(r["tflops"], 2) for v, r in results.items()},
         "mfma_util": {v: round(r["tflops"] / peak, 4) for v, r in results.items()},
+        "per_launch_us": spread,  # the reported variant, one event pair per launch
         "gemm_only_ms": round(gemm_mean, 5),
         "gemm_only_tflops": round(w.flop / (gemm_mean * 1e-3) / 1e12, 2),
         "roofline": {
