@@ -129,12 +129,10 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
-  __shared__ __attribute__((aligned(16))) char landing0[tccl::kBgSlotBytes];
-  __shared__ __attribute__((aligned(16))) char landing1[tccl::kBgSlotBytes];
   __shared__ __attribute__((aligned(16))) char landing_words[tccl::kBgWordBytes];
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
   tccl::Gemm256<InT, OutT, kWithReduce>(f.g, f.pull, (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
-                                        landing0, landing1, landing_words)
+                                        landing_words)
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();
   const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));

@@ -115,9 +115,9 @@ struct ReduceArgs {
 // loop (TileGroup variant): out[block of peer] <- the peer's copy of that block.
 // A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
 // pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
-// contiguous stretch.  At the start of a K step a wavefront fetches its next piece straight
-// into an LDS landing slot; behind the step's barrier (where its loads have landed) it reads
-// the piece into registers, and at the end of the step, behind the MFMAs, it stores it.  A
+// contiguous stretch.  At the start of a K step a wavefront requests its next piece into four
+// registers; the step's barrier waits for this wave's loads anyway, and mid-way through the
+// following step, away from the loads at a step's start, the piece is stored.  A
 // piece is fetched only once
 // the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
 // tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
@@ -147,7 +147,6 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
 };
-constexpr int kBgSlotBytes = 8 * 1024;                  // one 1 KiB landing slot per wavefront (there are two such arrays)
 constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter word per wavefront (64 lanes x 4 B)
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
@@ -200,11 +199,7 @@ struct Gemm256 {
   // are tracked per LDS variable, so a read of one stage need not wait for a load into the other.
   char* lds;   // stage 0 (also the epilogue's staging area)
   char* lds1;  // stage 1
-  // Landing area of the background transfer: one array per slot parity and one for the fetched
-  // counter words, so that a read of one need not wait for a fetch into another.
-  char* bg;    // slot 0 of every wavefront
-  char* bg1;   // slot 1
-  char* bgw;   // counter words
+  char* bgw;   // landing words of the background transfer's counter fetches
   const int tid, lane, wave, wm, wn;
   // A per-lane value the optimiser must treat as new at this point (blocks hoisting of what is derived from it).
   static TCCL_D int fresh(int v) {
@@ -213,8 +208,8 @@ struct Gemm256 {
   }
 
   TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, int reduce_args_offset, char* stage0,
-                 char* stage1, char* landing0, char* landing1 = nullptr, char* landing_words = nullptr)
-      : g(args), pa(pull_args), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bg(landing0), bg1(landing1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+                 char* stage1, char* landing_words)
+      : g(args), pa(pull_args), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
         wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
@@ -368,16 +363,13 @@ struct Gemm256 {
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
-    int pending_lp[2];       // per landing slot: the piece fetched into it and not yet stored (-1: none)
+    int pending_lp[2];       // per slot (K step parity): the piece requested into it and not yet stored (-1: none)
     int64_t pending_dst[2];  // and the destination block's address
-    int lds_off;             // this wavefront's landing slots inside the landing array
-    int probe_off;           // and its counter landing words
-    // What pull_collect() read out of the landing area right behind a K step's barrier: the
-    // counter word and the piece fetched at the step's start.  Read there, they are older than
-    // every operand fetch that follows, so using them later never waits for those.
+    u32x4 piece[2];          // the pieces themselves (slots are always named statically)
+    int probe_off;           // this wavefront's counter landing words
+    // The counter word, read out of the landing words right behind a K step's barrier: read
+    // there, it is older than every operand fetch that follows, so using it never waits for those.
     int32_t probe_val;
-    u32x4 piece;
-    int piece_slot;          // landing slot `piece` was read from (-1: none)
     // What the per-step code needs from PullArgs, kept in registers (reading a field through
     // the argument block is a scalar load plus a wait that also drains the operand fetches),
     // and piece positions that advance without divisions.
@@ -404,7 +396,6 @@ struct Gemm256 {
   TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
     PullState st;
     const int w = uniform(wave);
-    st.lds_off = w * 1024;
     st.probe_off = w * 256;
     st.stride = num_wgs * (kThreads256 / 64);
     st.next_slot = 0;
@@ -421,8 +412,7 @@ struct Gemm256 {
     st.pending_lp[0] = st.pending_lp[1] = -1;
     st.pending_dst[0] = st.pending_dst[1] = 0;
     st.probe_val = 0;
-    st.piece = u32x4{0, 0, 0, 0};
-    st.piece_slot = -1;
+    st.piece[0] = st.piece[1] = u32x4{0, 0, 0, 0};
     st.active = a.mode != kBgNone;
     st.primed = false;
     st.upr = st.pitch = st.units = 0;
@@ -491,8 +481,6 @@ struct Gemm256 {
   }
 
   // Row and 16-byte unit inside the row of this lane's unit of piece lp (row 0, unit 0 for idle lanes).
-  TCCL_D char* slot_ptr(const PullState& st, int slot) const { return (slot ? bg1 : bg) + st.lds_off; }
-
   TCCL_D void pull_unit(const PullArgs& a, int lp, bool& valid, uint32_t& row, uint32_t& col) const {
     const uint32_t u = (uint32_t)lp * 64u + (uint32_t)lane;
     valid = u < a.units;
@@ -546,16 +534,11 @@ struct Gemm256 {
     }
   }
 
-  // Store the piece sitting in landing slot `slot`, if any.  Returns whether a store was issued.
+  // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.
   TCCL_D bool pull_retire(PullState& st, const PullArgs& a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
     if (!st.active || st.pending_lp[slot] < 0) return false;
-    u32x4 v;
-    if (st.piece_slot == slot)
-      v = st.piece;  // already taken out of the landing slot by pull_collect()
-    else
-      v = *(const u32x4*)(slot_ptr(st, slot) + lane * 16);
-    st.piece_slot = -1;
+    const u32x4 v = st.piece[slot];
     // The store must use the bases of the block the piece belongs to: pieces are retired
     // before the slot selection moves on (pull_issue), except for the one in flight when it
     // does, whose bases are kept aside.
@@ -577,21 +560,16 @@ struct Gemm256 {
     pull_group_facts(st, a);
   }
 
-  // Start of a K step: learn about readiness, fetch the next piece into landing slot `slot`
-  // (its previous piece was stored at the end of the step before last).  All control flow
-  // here is wavefront-uniform.
-  // Right behind a K step's barrier (this wave's loads, the background fetches among them,
-  // have landed): take the counter word and the piece fetched into `slot` at the step's start
-  // out of the landing area.
+  // Right behind a K step's barrier (this wave's loads, the counter fetch among them, have
+  // landed): take the counter word out of the landing words.
   TCCL_D void pull_collect(PullState& st, const PullArgs& a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return;
     if (!st.active) return;
     st.probe_val = *(const int32_t*)(bgw + st.probe_off);
-    if (st.pending_lp[slot] >= 0) {
-      st.piece = *(const u32x4*)(slot_ptr(st, slot) + lane * 16);
-      st.piece_slot = slot;
-    }
   }
+  // Start of a K step: learn about readiness, request the next piece into slot `slot` (its
+  // previous piece was stored during the step before).  All control flow here is
+  // wavefront-uniform.  Returns whether a piece was requested.
   TCCL_D bool pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
     if (!st.active) return false;
@@ -617,8 +595,7 @@ struct Gemm256 {
     if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
       const bool valid = (uint32_t)st.next_lp * 64u + (uint32_t)lane < st.units;
       const uint32_t off = valid ? st.row * st.pitch + st.col * 16u : 0u;  // idle lanes touch the block's first unit
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(window(st.src_base), (LdsVoid*)slot_ptr(st, slot), 16, off, 0, 0,
-                                               kCoherent);
+      st.piece[slot] = ld16<kCoherent>(window(st.src_base), off);
       st.pending_lp[slot] = st.next_lp;
       st.pending_dst[slot] = st.dst_base;
       st.pend_off[slot] = off;
@@ -735,7 +712,7 @@ struct Gemm256 {
   // 4096^3 e4m3: 54 us against 62 us with the barrier at the step's end.
   TCCL_D void k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                       Frags8& f, PullState& pull, int parity) const {
-    pull_issue(pull, pa, bg, parity);
+    pull_issue(pull, pa, bgw, parity);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int kk = i >> 2, bi = i & 3;
@@ -744,7 +721,7 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        pull_collect(pull, pa, bg, parity);
+        pull_collect(pull, pa, bgw, parity);
       }
       const char* from = i + 1 < 8 ? cur : nxt;
       f.ring[(i + 1) & 1] = load_a8(from, rd, j >> 2, j & 3);
@@ -761,7 +738,7 @@ struct Gemm256 {
       acc[bi][1] = Mfma<InT>::run(f.fb[kk][1], f.ring[i & 1], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    pull_retire(pull, pa, bg, parity);  // the piece this step fetched, collected behind the barrier
+    pull_retire(pull, pa, bgw, parity);  // the piece this step requested: it arrived before the barrier
   }
 
   // One K step of the 16-bit path: sixteen items (k-block kk, A slab bi) of two MFMAs each,
@@ -785,7 +762,7 @@ struct Gemm256 {
   // issues meanwhile; later or denser placements measured slower.
   TCCL_D void k_step16(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                        Frags& f, PullState& pull, int parity) const {
-    pull_issue(pull, pa, bg, parity);
+    pull_issue(pull, pa, bgw, parity);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int kk = i >> 2, bi = i & 3;
@@ -797,16 +774,17 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        pull_collect(pull, pa, bg, parity);
+        pull_collect(pull, pa, bgw, parity);
       }
       const char* from = i + 2 < 16 ? cur : nxt;
       if ((j & 3) == 0) load_b16(from, rd, j >> 2, f.fbr[(j >> 2) & 1]);
       f.ring[(i + 2) & 3] = load_a16(from, rd, j >> 2, j & 3);
       if (i < 8 && (i & 1) == 0) issue_piece(nxt, src, kt_load, i >> 1);
-      // The piece of the step before (collected behind that step's barrier) is stored here,
-      // away from the cluster of loads at the step's start: 1.8 % on the all-gather at
-      // 4096x4096x1024 against storing it at the end of its own step.
-      if (i == 9) pull_retire(pull, pa, bg, parity ^ 1);
+      // The piece requested at the start of the step before (it arrived before that step's
+      // barrier) is stored here, away from the cluster of loads at a step's start: 0.4-1.8 %
+      // on the all-gather at 4096x4096x1024 against storing it at the end of its own step,
+      // 1.6 % against storing it right behind the barrier.
+      if (i == 9) pull_retire(pull, pa, bgw, parity ^ 1);
       acc[bi][0] = Mfma<InT>::run(f.fbr[kk & 1][0], f.ring[i & 3], acc[bi][0]);
       acc[bi][1] = Mfma<InT>::run(f.fbr[kk & 1][1], f.ring[i & 3], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -1038,13 +1016,13 @@ struct Gemm256 {
     // The first counters are requested behind the first operands: the chain of dependent
     // scalar loads that leads to them (slice bases, tile counts) then runs while those are in flight.
     if (!pull.primed) {
-      pull_prime(pull, pa, bg);
+      pull_prime(pull, pa, bgw);
       pull.primed = true;
     }
     wait_vmem();  // the first operands are there, and so is everything the previous tile stored
     __syncthreads();
     publish_owed(s, unpublished);
-    pull_collect(pull, pa, bg, 0);  // the counters fetched before this tile (no piece is pending here)
+    pull_collect(pull, pa, bgw, 0);  // the counters fetched before this tile (no piece is pending here)
     if constexpr (kFp8) {
       Frags8 f;
       f.fb[0][0] = load_b8(lds, rd, 0, 0);
@@ -1063,7 +1041,7 @@ struct Gemm256 {
         k_step16(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
         k_step16(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
-      pull_retire(pull, pa, bg, 1);  // the last step's piece: nothing is carried through the epilogue
+      pull_retire(pull, pa, bgw, 1);  // the last step's piece: nothing is carried through the epilogue
     }
     if constexpr (kWithReduce) {
       // Rows this rank owns, partial kept in registers: the peers' partials are added in the
@@ -1278,7 +1256,7 @@ struct Gemm256 {
       __syncthreads();
       publish_owed(s, unpublished);
     }
-    pull_finish(pull, pa, bg, num_wgs);
+    pull_finish(pull, pa, bgw, num_wgs);
   }
 };
 #endif  // __HIP_DEVICE_COMPILE__
