@@ -115,9 +115,9 @@ struct ReduceArgs {
 // loop (TileGroup variant): out[block of peer] <- the peer's copy of that block.
 // A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
 // pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
-// contiguous stretch.  At the start of a K step a wavefront requests its next piece into four
-// registers; the step's barrier waits for this wave's loads anyway, and mid-way through the
-// following step, away from the loads at a step's start, the piece is stored.  A
+// contiguous stretch.  In every K step, behind the step's operand loads, a wavefront requests
+// its next piece into four registers; the step's barrier waits for this wave's loads anyway,
+// and mid-way through the following step the piece is stored.  A
 // piece is fetched only once
 // the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
 // tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
@@ -567,7 +567,7 @@ struct Gemm256 {
     if (!st.active) return;
     st.probe_val = *(const int32_t*)(bgw + st.probe_off);
   }
-  // Start of a K step: learn about readiness, request the next piece into slot `slot` (its
+  // Once per K step: learn about readiness, request the next piece into slot `slot` (its
   // previous piece was stored during the step before).  All control flow here is
   // wavefront-uniform.  Returns whether a piece was requested.
   TCCL_D bool pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
@@ -762,7 +762,6 @@ struct Gemm256 {
   // issues meanwhile; later or denser placements measured slower.
   TCCL_D void k_step16(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                        Frags& f, PullState& pull, int parity) const {
-    pull_issue(pull, pa, bgw, parity);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int kk = i >> 2, bi = i & 3;
@@ -785,6 +784,11 @@ struct Gemm256 {
       // on the all-gather at 4096x4096x1024 against storing it at the end of its own step,
       // 1.6 % against storing it right behind the barrier.
       if (i == 9) pull_retire(pull, pa, bgw, parity ^ 1);
+      // The next piece is requested behind the step's last operand loads, not ahead of them:
+      // loads complete in issue order, so a request that has to go out to the peer's memory
+      // would hold back every operand load issued after it (2.4 % on the same workload
+      // against requesting it at the step's start).
+      if (i == 7) pull_issue(pull, pa, bgw, parity);
       acc[bi][0] = Mfma<InT>::run(f.fbr[kk & 1][0], f.ring[i & 3], acc[bi][0]);
       acc[bi][1] = Mfma<InT>::run(f.fbr[kk & 1][1], f.ring[i & 3], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
