@@ -99,6 +99,7 @@ __global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl:
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
+  tccl::warm_kernargs<(int)(sizeof(tccl::GemmArgs) + sizeof(tccl::Macro))>();
   tccl::SignalArgs s;
   s.mode = tccl::kSignalNone;
   tccl::PullArgs no_pull = {};  // mode 0: no background transfer
@@ -130,6 +131,7 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
   __shared__ __attribute__((aligned(16))) char landing_words[tccl::kBgWordBytes];
+  tccl::warm_kernargs<(int)sizeof(Fused256Args)>();
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
   tccl::Gemm256<InT, OutT, kWithReduce>(f.g, f.pull, (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
                                         landing_words)

@@ -181,6 +181,20 @@ TCCL_D T late_kernarg(int offset) {
   return v;
 }
 
+// Request every 64-byte line of the kernel arguments at once.  The compiler reads arguments
+// where it first needs them, each group of reads followed by its own wait, so a kernel's
+// start used to be a chain of a dozen dependent trips to memory before the first operand load
+// could go out; after this the later reads hit in the scalar cache.
+template <int kBytes>
+TCCL_D void warm_kernargs() {
+  typedef const __attribute__((address_space(4))) uint32_t* Words;
+  Words p = (Words)__builtin_amdgcn_kernarg_segment_ptr();
+  uint32_t any = 0;
+#pragma unroll
+  for (int o = 0; o < kBytes; o += 64) any |= p[o / 4];
+  asm volatile("" ::"s"(any));
+}
+
 template <typename InT, typename OutT, bool kWithReduce = false>
 struct Gemm256 {
   typedef typename Mfma<InT>::Vec Vec;
@@ -1241,15 +1255,20 @@ struct Gemm256 {
     }
   }
 
+  static TCCL_D TileCoord tile_of_slot(int slot, int total, const Macro& m) {
+    const int id = tile_for_slot(slot, total, m.xcds, m.span);
+    TileCoord c = macro_coords(id, m);
+    c.m += m.row_shift;
+    if (c.m >= m.rows) c.m -= m.rows;
+    return c;
+  }
+
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
     const int total = m.rows * m.cols;
     PullState pull = pull_begin(pa, wg, num_wgs);
     int unpublished = -1;
     for (int slot = wg; slot < total; slot += num_wgs) {
-      const int id = tile_for_slot(slot, total, m.xcds, m.span);
-      TileCoord c = macro_coords(id, m);
-      c.m += m.row_shift;
-      if (c.m >= m.rows) c.m -= m.rows;
+      const TileCoord c = tile_of_slot(slot, total, m);
       if (s.mode == kSignalNone && push_offset < 0)
         macro_tile<0>(s, c.m, c.n, pull, unpublished);
       else
