@@ -102,8 +102,7 @@ __global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl:
   tccl::warm_kernargs<(int)(sizeof(tccl::GemmArgs) + sizeof(tccl::Macro))>();
   tccl::SignalArgs s;
   s.mode = tccl::kSignalNone;
-  tccl::PullArgs no_pull = {};  // mode 0: no background transfer
-  tccl::Gemm256<InT, OutT>(g, no_pull, -1, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
+  tccl::Gemm256<InT, OutT>(g, -1, -1, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
 #endif
 }
 
@@ -133,7 +132,7 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
   __shared__ __attribute__((aligned(16))) char landing_words[tccl::kBgWordBytes];
   tccl::warm_kernargs<(int)sizeof(Fused256Args)>();
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
-  tccl::Gemm256<InT, OutT, kWithReduce>(f.g, f.pull, (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
+  tccl::Gemm256<InT, OutT, kWithReduce>(f.g, (int)offsetof(Fused256Args, pull), (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
                                         landing_words)
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();

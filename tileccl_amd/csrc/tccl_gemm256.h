@@ -206,7 +206,11 @@ struct Gemm256 {
   static constexpr bool kFp8 = kEszIn == 1;
 
   const GemmArgs& g;
-  const PullArgs& pa;
+  // Byte offset of a PullArgs in the kernel arguments (< 0: no background transfer).  Like the
+  // push and reduce arguments it is read where it is used: taken as a kernel argument struct its
+  // thirty-odd fields were loaded at the kernel's start and held in scalar registers (or the
+  // lanes they spill to) through every K loop.
+  const int pull_offset;
   const int push_offset;    // byte offset of a PushArgs in the kernel arguments; < 0: no push
   const int reduce_offset;  // byte offset of a ReduceArgs in the kernel arguments; < 0: none
   // The two pipeline stages are two separate __shared__ arrays: loads that write LDS directly
@@ -221,12 +225,14 @@ struct Gemm256 {
     return v;
   }
 
-  TCCL_D Gemm256(const GemmArgs& args, const PullArgs& pull_args, int push_args_offset, int reduce_args_offset, char* stage0,
+  TCCL_D Gemm256(const GemmArgs& args, int pull_args_offset, int push_args_offset, int reduce_args_offset, char* stage0,
                  char* stage1, char* landing_words)
-      : g(args), pa(pull_args), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
         wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
+  typedef const __attribute__((address_space(4))) PullArgs* PullPtr;
+  TCCL_D PullPtr pa() const { return late_kernarg_ptr<PullArgs>(pull_offset < 0 ? 0 : pull_offset); }
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   typedef short s16x8 __attribute__((ext_vector_type(8)));
   typedef __attribute__((address_space(3))) s16x4 LdsQuad;
@@ -407,7 +413,7 @@ struct Gemm256 {
     return ((const __attribute__((address_space(4))) T*)p)[i];
   }
 
-  TCCL_D PullState pull_begin(const PullArgs& a, int wg, int num_wgs) const {
+  TCCL_D PullState pull_begin(PullPtr a, int wg, int num_wgs) const {
     PullState st;
     const int w = uniform(wave);
     st.probe_off = w * 256;
@@ -427,7 +433,7 @@ struct Gemm256 {
     st.pending_dst[0] = st.pending_dst[1] = 0;
     st.probe_val = 0;
     st.piece[0] = st.piece[1] = u32x4{0, 0, 0, 0};
-    st.active = a.mode != kBgNone;
+    st.active = pull_offset >= 0 && a->mode != kBgNone;
     st.primed = false;
     st.upr = st.pitch = st.units = 0;
     st.pieces = st.slots = st.n_groups = 0;
@@ -435,12 +441,12 @@ struct Gemm256 {
     st.pend_off[0] = st.pend_off[1] = 0;
     st.pend_valid[0] = st.pend_valid[1] = false;
     if (st.active) {
-      st.upr = a.upr;
-      st.pitch = a.pitch;
-      st.units = a.units;
-      st.pieces = a.pieces;
-      st.slots = a.slots;
-      st.n_groups = a.n_groups;
+      st.upr = a->upr;
+      st.pitch = a->pitch;
+      st.units = a->units;
+      st.pieces = a->pieces;
+      st.slots = a->slots;
+      st.n_groups = a->n_groups;
       const uint32_t adv = (uint32_t)st.stride * 64u;
       st.adv_row = adv / st.upr;
       st.adv_col = adv - st.adv_row * st.upr;
@@ -468,15 +474,15 @@ struct Gemm256 {
 
   // Fetch the first counters in the first tile's prologue, so that the first K step can
   // already fetch a piece.
-  TCCL_D void pull_prime(PullState& st, const PullArgs& a, char* landing) const {
+  TCCL_D void pull_prime(PullState& st, PullPtr a, char* landing) const {
     if constexpr (kWithReduce) return;  // that instantiation never pulls: its launch clears PullArgs
-    if (a.mode == kBgNone || st.next_slot >= a.slots) return;
+    if (!st.active || st.next_slot >= a->slots) return;
     pull_select(st, a, st.next_slot);
     pull_probe(st, a, landing);
   }
 
   // Every lane fetches the same word; it is read back from LDS one K step later.
-  TCCL_D void pull_probe(PullState& st, const PullArgs& a, char* landing) const {
+  TCCL_D void pull_probe(PullState& st, PullPtr a, char* landing) const {
     if (st.gidx >= st.n_groups) return;
     if (st.backoff > 0) {
       --st.backoff;
@@ -487,40 +493,40 @@ struct Gemm256 {
     st.probe_group = st.gidx;
   }
 
-  TCCL_D void pull_normalise(PullState& st, const PullArgs& a) const {
-    while (st.next_lp >= a.pieces && st.next_slot < a.slots) {
-      st.next_lp -= a.pieces;
+  TCCL_D void pull_normalise(PullState& st, PullPtr a) const {
+    while (st.next_lp >= a->pieces && st.next_slot < a->slots) {
+      st.next_lp -= a->pieces;
       ++st.next_slot;
     }
   }
 
   // Row and 16-byte unit inside the row of this lane's unit of piece lp (row 0, unit 0 for idle lanes).
-  TCCL_D void pull_unit(const PullArgs& a, int lp, bool& valid, uint32_t& row, uint32_t& col) const {
+  TCCL_D void pull_unit(PullPtr a, int lp, bool& valid, uint32_t& row, uint32_t& col) const {
     const uint32_t u = (uint32_t)lp * 64u + (uint32_t)lane;
-    valid = u < a.units;
+    valid = u < a->units;
     const uint32_t uu = valid ? u : 0u;  // idle lanes touch the block's first unit and store nothing
-    row = uu / a.upr;
-    col = uu - row * a.upr;
+    row = uu / a->upr;
+    col = uu - row * a->upr;
   }
 
-  TCCL_D uint32_t pull_last_unit(const PullArgs& a, int lp) const {
+  TCCL_D uint32_t pull_last_unit(PullPtr a, int lp) const {
     const uint32_t last = (uint32_t)lp * 64u + 63u;
-    return last < a.units ? last : a.units - 1u;
+    return last < a->units ? last : a->units - 1u;
   }
 
-  TCCL_D void pull_select(PullState& st, const PullArgs& a, int slot) const {
+  TCCL_D void pull_select(PullState& st, PullPtr a, int slot) const {
     if (slot == st.slot) return;
     st.slot = slot;
     st.ready_units = 0;
     st.probe_group = -1;
     st.backoff = 0;
-    const int64_t mine = table(a.heap_bases, a.rank);
-    const int peer = slot < a.rank ? slot : slot + 1;
-    const int64_t theirs = table(a.heap_bases, peer);
-    const int64_t rel = ((int64_t)(uintptr_t)a.src0 - mine) + (int64_t)peer * a.block_bytes;
+    const int64_t mine = table(a->heap_bases, a->rank);
+    const int peer = slot < a->rank ? slot : slot + 1;
+    const int64_t theirs = table(a->heap_bases, peer);
+    const int64_t rel = ((int64_t)(uintptr_t)a->src0 - mine) + (int64_t)peer * a->block_bytes;
     st.src_base = theirs + rel;
     st.dst_base = mine + rel;
-    st.counter_base = (int64_t)(uintptr_t)a.counter + (theirs - mine);
+    st.counter_base = (int64_t)(uintptr_t)a->counter + (theirs - mine);
     st.row0 = 0;  // the plan numbers the rows of one block
     st.gidx = 0;
     pull_group_facts(st, a);
@@ -549,7 +555,7 @@ struct Gemm256 {
   }
 
   // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.
-  TCCL_D bool pull_retire(PullState& st, const PullArgs& a, const char* landing, int slot) const {
+  TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
     if (!st.active || st.pending_lp[slot] < 0) return false;
     const u32x4 v = st.piece[slot];
@@ -563,12 +569,12 @@ struct Gemm256 {
   }
 
   // The two facts about group gidx that the per-step code needs, fetched when gidx changes.
-  TCCL_D void pull_group_facts(PullState& st, const PullArgs& a) const {
-    if (st.gidx >= a.n_groups) return;
-    st.need = a.epoch * table(a.tile_counts, st.gidx);
-    st.group_units = (uint32_t)(table(a.row_ends, st.gidx) - st.row0) * a.upr;
+  TCCL_D void pull_group_facts(PullState& st, PullPtr a) const {
+    if (st.gidx >= a->n_groups) return;
+    st.need = a->epoch * table(a->tile_counts, st.gidx);
+    st.group_units = (uint32_t)(table(a->row_ends, st.gidx) - st.row0) * a->upr;
   }
-  TCCL_D void pull_group_done(PullState& st, const PullArgs& a) const {
+  TCCL_D void pull_group_done(PullState& st, PullPtr a) const {
     st.ready_units = st.group_units;
     ++st.gidx;
     pull_group_facts(st, a);
@@ -576,7 +582,7 @@ struct Gemm256 {
 
   // Right behind a K step's barrier (this wave's loads, the counter fetch among them, have
   // landed): take the counter word out of the landing words.
-  TCCL_D void pull_collect(PullState& st, const PullArgs& a, const char* landing, int slot) const {
+  TCCL_D void pull_collect(PullState& st, PullPtr a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return;
     if (!st.active) return;
     st.probe_val = *(const int32_t*)(bgw + st.probe_off);
@@ -584,7 +590,7 @@ struct Gemm256 {
   // Once per K step: learn about readiness, request the next piece into slot `slot` (its
   // previous piece was stored during the step before).  All control flow here is
   // wavefront-uniform.  Returns whether a piece was requested.
-  TCCL_D bool pull_issue(PullState& st, const PullArgs& a, char* landing, int slot) const {
+  TCCL_D bool pull_issue(PullState& st, PullPtr a, char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
     if (!st.active) return false;
     if (st.probe_group >= 0) {
@@ -627,9 +633,9 @@ struct Gemm256 {
   }
 
   // Wait (bounded) until units [0, last] of the selected block may be fetched.
-  TCCL_D bool pull_wait_ready(PullState& st, const PullArgs& a, uint32_t last, int64_t deadline) const {
+  TCCL_D bool pull_wait_ready(PullState& st, PullPtr a, uint32_t last, int64_t deadline) const {
     while (last >= st.ready_units) {
-      if (st.gidx >= a.n_groups) return false;
+      if (st.gidx >= a->n_groups) return false;
       const int32_t need = st.need;
       const __amdgpu_buffer_rsrc_t words = window(st.counter_base);
       for (;;) {
@@ -644,17 +650,17 @@ struct Gemm256 {
   }
 
   // After the last tile: finish what is in flight, move the remaining pieces, report.
-  TCCL_D void pull_finish(PullState& st, const PullArgs& a, const char* landing, int num_wgs) const {
+  TCCL_D void pull_finish(PullState& st, PullPtr a, const char* landing, int num_wgs) const {
     if constexpr (kWithReduce) return;
-    if (a.mode == kBgNone) return;
+    if (!st.active) return;
     wait_vmem();
     pull_retire(st, a, landing, 0);
     pull_retire(st, a, landing, 1);
     st.probe_group = -1;
-    const int64_t deadline = now_ticks() + a.spin_ticks;
+    const int64_t deadline = now_ticks() + a->spin_ticks;
     bool ok = true;
     constexpr int kBatch = 8;  // pieces in flight per wavefront: the CU has no other work left
-    while (ok && st.next_slot < a.slots) {
+    while (ok && st.next_slot < a->slots) {
       pull_select(st, a, st.next_slot);
       u32x4 v[kBatch];
       uint32_t row[kBatch], col[kBatch];
@@ -664,11 +670,11 @@ struct Gemm256 {
       for (int k = 0; k < kBatch; ++k) {
         valid[k] = loaded[k] = false;
         const int lp = st.next_lp + k * st.stride;
-        if (ok && lp < a.pieces) {
+        if (ok && lp < a->pieces) {
           ok = pull_wait_ready(st, a, pull_last_unit(a, lp), deadline);
           if (ok) {
             pull_unit(a, lp, valid[k], row[k], col[k]);
-            const uint32_t off = row[k] * a.pitch + col[k] * 16u;
+            const uint32_t off = row[k] * a->pitch + col[k] * 16u;
             v[k] = ld16<kCoherent>(window(st.src_base), off);
             loaded[k] = true;
             n = k + 1;
@@ -677,17 +683,17 @@ struct Gemm256 {
       }
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
-        if (loaded[k] && valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a.pitch + col[k] * 16u, v[k]);
+        if (loaded[k] && valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a->pitch + col[k] * 16u, v[k]);
       }
       st.next_lp += n * st.stride;
       if (n < kBatch) {  // the block is finished (or a wait gave up)
-        st.next_lp -= a.pieces;
+        st.next_lp -= a->pieces;
         if (st.next_lp < 0) st.next_lp = 0;  // only after a failed wait
         ++st.next_slot;
         pull_normalise(st, a);
       }
     }
-    if (!ok && lane == 0 && a.fault) *a.fault = 1;
+    if (!ok && lane == 0 && a->fault) *a->fault = 1;
     wait_vmem();
     __syncthreads();
     // Only a traced launch counts arrivals: one per workgroup on barrier[0], and the last one
@@ -695,12 +701,12 @@ struct Gemm256 {
     // Nobody waits on these words (a pull completes on the pulling rank, whose kernel ends;
     // pushes are announced by counter[g]), and 256 adds to one word cost ~7 ns each here,
     // ~1 us at the very end of every launch.
-    if (tid == 0 && a.barrier && a.trace_done_clock) {
-      const int32_t prev = tile_signal_add<true>(a.barrier, 0, 1);
-      if (prev + 1 == a.epoch * num_wgs) {
-        for (int g = 0; g < a.n_groups; ++g) {
-          if (g > 0) tile_signal_add<true>(a.barrier, g, num_wgs);
-          a.trace_done_clock[g] = now_ticks();
+    if (tid == 0 && a->barrier && a->trace_done_clock) {
+      const int32_t prev = tile_signal_add<true>(a->barrier, 0, 1);
+      if (prev + 1 == a->epoch * num_wgs) {
+        for (int g = 0; g < a->n_groups; ++g) {
+          if (g > 0) tile_signal_add<true>(a->barrier, g, num_wgs);
+          a->trace_done_clock[g] = now_ticks();
         }
       }
     }
@@ -726,7 +732,7 @@ struct Gemm256 {
   // 4096^3 e4m3: 54 us against 62 us with the barrier at the step's end.
   TCCL_D void k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                       Frags8& f, PullState& pull, int parity) const {
-    pull_issue(pull, pa, bgw, parity);
+    pull_issue(pull, pa(), bgw, parity);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int kk = i >> 2, bi = i & 3;
@@ -735,7 +741,7 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        pull_collect(pull, pa, bgw, parity);
+        pull_collect(pull, pa(), bgw, parity);
       }
       const char* from = i + 1 < 8 ? cur : nxt;
       f.ring[(i + 1) & 1] = load_a8(from, rd, j >> 2, j & 3);
@@ -752,7 +758,7 @@ struct Gemm256 {
       acc[bi][1] = Mfma<InT>::run(f.fb[kk][1], f.ring[i & 1], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    pull_retire(pull, pa, bgw, parity);  // the piece this step requested: it arrived before the barrier
+    pull_retire(pull, pa(), bgw, parity);  // the piece this step requested: it arrived before the barrier
   }
 
   // One K step of the 16-bit path: sixteen items (k-block kk, A slab bi) of two MFMAs each,
@@ -787,7 +793,7 @@ struct Gemm256 {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        pull_collect(pull, pa, bgw, parity);
+        pull_collect(pull, pa(), bgw, parity);
       }
       const char* from = i + 2 < 16 ? cur : nxt;
       if ((j & 3) == 0) load_b16(from, rd, j >> 2, f.fbr[(j >> 2) & 1]);
@@ -797,12 +803,12 @@ struct Gemm256 {
       // barrier) is stored here, away from the cluster of loads at a step's start: 0.4-1.8 %
       // on the all-gather at 4096x4096x1024 against storing it at the end of its own step,
       // 1.6 % against storing it right behind the barrier.
-      if (i == 9) pull_retire(pull, pa, bgw, parity ^ 1);
+      if (i == 9) pull_retire(pull, pa(), bgw, parity ^ 1);
       // The next piece is requested behind the step's last operand loads, not ahead of them:
       // loads complete in issue order, so a request that has to go out to the peer's memory
       // would hold back every operand load issued after it (2.4 % on the same workload
       // against requesting it at the step's start).
-      if (i == 7) pull_issue(pull, pa, bgw, parity);
+      if (i == 7) pull_issue(pull, pa(), bgw, parity);
       acc[bi][0] = Mfma<InT>::run(f.fbr[kk & 1][0], f.ring[i & 3], acc[bi][0]);
       acc[bi][1] = Mfma<InT>::run(f.fbr[kk & 1][1], f.ring[i & 3], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -1034,13 +1040,13 @@ struct Gemm256 {
     // The first counters are requested behind the first operands: the chain of dependent
     // scalar loads that leads to them (slice bases, tile counts) then runs while those are in flight.
     if (!pull.primed) {
-      pull_prime(pull, pa, bgw);
+      pull_prime(pull, pa(), bgw);
       pull.primed = true;
     }
     wait_vmem();  // the first operands are there, and so is everything the previous tile stored
     __syncthreads();
     publish_owed(s, unpublished);
-    pull_collect(pull, pa, bgw, 0);  // the counters fetched before this tile (no piece is pending here)
+    pull_collect(pull, pa(), bgw, 0);  // the counters fetched before this tile (no piece is pending here)
     if constexpr (kFp8) {
       Frags8 f;
       f.fb[0][0] = load_b8(lds, rd, 0, 0);
@@ -1059,7 +1065,7 @@ struct Gemm256 {
         k_step16(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
         k_step16(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
-      pull_retire(pull, pa, bgw, 1);  // the last step's piece: nothing is carried through the epilogue
+      pull_retire(pull, pa(), bgw, 1);  // the last step's piece: nothing is carried through the epilogue
     }
     if constexpr (kWithReduce) {
       // Rows this rank owns, partial kept in registers: the peers' partials are added in the
@@ -1265,7 +1271,7 @@ struct Gemm256 {
 
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
     const int total = m.rows * m.cols;
-    PullState pull = pull_begin(pa, wg, num_wgs);
+    PullState pull = pull_begin(pa(), wg, num_wgs);
     int unpublished = -1;
     for (int slot = wg; slot < total; slot += num_wgs) {
       const TileCoord c = tile_of_slot(slot, total, m);
@@ -1279,7 +1285,7 @@ struct Gemm256 {
       __syncthreads();
       publish_owed(s, unpublished);
     }
-    pull_finish(pull, pa, bgw, num_wgs);
+    pull_finish(pull, pa(), bgw, num_wgs);
   }
 };
 #endif  // __HIP_DEVICE_COMPILE__
