@@ -107,6 +107,42 @@ def test_fp8_reduce_scatter_two_ranks(lib, variant):
             h.cleanup()
 
 
+@pytest.mark.parametrize("variant", ["s0", "s1", "s2"])
+@pytest.mark.parametrize("directions", ["both", "pull"])
+def test_fp8_allgather_two_ranks(lib, variant, directions):
+    """GEMM-output AllGather with e4m3 inputs and a bf16 output: the fp8 K loop carries the
+    background pull of S2 (a few pieces per wavefront inside the K loop, the rest after the
+    last tile).  The product is held to the fp8 tolerance, everything moved is bit-exact."""
+    from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+    M, N, K = 1024, 512, 512
+    heaps = SymmetricHeap.create_all(64 << 20, 2)
+    try:
+        ops = [FusedGemmAllGather(h, M, N, torch.bfloat16, directions=directions) for h in heaps]
+        op = ops[0]
+        A_cpu, sa = quantise((M, K), 0)
+        B_cpu, sb = quantise((K, N), 1, K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        block = seeded((M, N), 2, torch.bfloat16)
+        for o in ops:
+            o.out.zero_()
+        ops[1].out[M:].copy_(block)
+        op.mark_peers_ready()
+        op(A, B, variant, scale_a=sa, scale_b=sb)
+        op.check_faults()
+        mine = op.out[:M].clone()
+        assert_gemm_close(mine, (A_cpu.float() @ B_cpu.float()) * (sa * sb), rtol=5e-2, tight=0.032)
+        if directions == "both":
+            assert torch.equal(bits(op.peer_out(1)[:M]), bits(mine))
+        else:
+            assert torch.count_nonzero(op.peer_out(1)[:M]).item() == 0  # nothing pushed
+        assert torch.equal(bits(op.out[M:]).cpu(), bits(block))  # the pulled block
+        assert torch.equal(bits(op.peer_out(1)[M:]).cpu(), bits(block))  # the peer's own block is untouched
+    finally:
+        for h in heaps:
+            h.cleanup()
+
+
 def test_baseline_config_4_properties(lib):
     """16384x2048 @ 2048x4096 e4m3 with per-tensor scales, resident bf16 peer partial: the three
     variants agree byte for byte, the reduction equals the oracle on slabs of both owners, the
