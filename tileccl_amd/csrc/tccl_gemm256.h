@@ -383,8 +383,7 @@ struct Gemm256 {
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
-    int pending_lp[2];       // per slot (K step parity): the piece requested into it and not yet stored (-1: none)
-    int64_t pending_dst[2];  // and the destination block's address
+    int pend_mask;           // bit per slot (K step parity): a piece was requested into it and is not yet stored
     u32x4 piece[2];          // the pieces themselves (slots are always named statically)
     int probe_off;           // this wavefront's counter landing words
     // The counter word, read out of the landing words right behind a K step's barrier: read
@@ -399,8 +398,8 @@ struct Gemm256 {
     int pieces, slots, n_groups;
     uint32_t adv_row, adv_col;   // what `stride` pieces add to (row, col)
     uint32_t row, col;           // per lane: row / unit of this lane's unit of piece next_lp
-    uint32_t pend_off[2];        // per lane: byte offset of the pending piece inside its block
-    bool pend_valid[2];          // per lane: the unit exists (the last piece of a block may be short)
+    uint32_t pend_off[2];        // per lane: byte offset of the pending piece inside its block; kNoUnit: the
+                                 // unit does not exist (the last piece of a block may be short)
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -429,8 +428,7 @@ struct Gemm256 {
     st.need = 0;
     st.group_units = 0;
     st.backoff = 0;
-    st.pending_lp[0] = st.pending_lp[1] = -1;
-    st.pending_dst[0] = st.pending_dst[1] = 0;
+    st.pend_mask = 0;
     st.probe_val = 0;
     st.piece[0] = st.piece[1] = u32x4{0, 0, 0, 0};
     st.active = pull_offset >= 0 && a->mode != kBgNone;
@@ -439,7 +437,6 @@ struct Gemm256 {
     st.pieces = st.slots = st.n_groups = 0;
     st.adv_row = st.adv_col = st.row = st.col = 0;
     st.pend_off[0] = st.pend_off[1] = 0;
-    st.pend_valid[0] = st.pend_valid[1] = false;
     if (st.active) {
       st.upr = a->upr;
       st.pitch = a->pitch;
@@ -554,17 +551,17 @@ struct Gemm256 {
     }
   }
 
-  // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.
+  static constexpr uint32_t kNoUnit = 0xffffffffu;
+
+  // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.  The
+  // piece belongs to the selected block: pull_issue() stores what is pending before it selects
+  // another one.
   TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
-    if (!st.active || st.pending_lp[slot] < 0) return false;
-    const u32x4 v = st.piece[slot];
-    // The store must use the bases of the block the piece belongs to: pieces are retired
-    // before the slot selection moves on (pull_issue), except for the one in flight when it
-    // does, whose bases are kept aside.
-    const int64_t dst = st.pending_dst[slot];
-    if (st.pend_valid[slot]) st16<kStreaming>(window(dst), st.pend_off[slot], v);
-    st.pending_lp[slot] = -1;
+    if (!(st.pend_mask & (1 << slot))) return false;
+    const uint32_t off = st.pend_off[slot];
+    if (off != kNoUnit) st16<kStreaming>(window(st.dst_base), off, st.piece[slot]);
+    st.pend_mask &= ~(1 << slot);
     return true;
   }
 
@@ -606,6 +603,7 @@ struct Gemm256 {
     }
     if (st.next_slot >= st.slots) return false;
     if (st.next_slot != st.slot) {
+      pull_retire(st, a, landing, slot ^ 1);  // the piece of the step before belongs to the block being left
       pull_select(st, a, st.next_slot);
       pull_probe(st, a, landing);
       return false;
@@ -616,10 +614,8 @@ struct Gemm256 {
       const bool valid = (uint32_t)st.next_lp * 64u + (uint32_t)lane < st.units;
       const uint32_t off = valid ? st.row * st.pitch + st.col * 16u : 0u;  // idle lanes touch the block's first unit
       st.piece[slot] = ld16<kCoherent>(window(st.src_base), off);
-      st.pending_lp[slot] = st.next_lp;
-      st.pending_dst[slot] = st.dst_base;
-      st.pend_off[slot] = off;
-      st.pend_valid[slot] = valid;
+      st.pend_off[slot] = valid ? off : kNoUnit;
+      st.pend_mask |= 1 << slot;
       st.next_lp += st.stride;
       if (st.next_lp >= st.pieces) {  // block finished: rare, may divide
         pull_normalise(st, a);
