@@ -104,22 +104,27 @@ typedef struct tccl_gemm_desc {
 /* ---- per-launch synchronisation words ------------------------------------------------
  * Stands in for the lock tensor of WGSpecializedPattern (wg_specialized.py:104-124) and
  * for TileGroupSignalState (tileccl_v2/signal.py:14-40).
- *   locks      int32[total_tiles]   S1: tile_signal / tile_wait (sync/primitives.py:357-414)
+ *   locks      int32[total_tiles]   S1: launch number `epoch` is stored per finished tile; a tile is ready
+ *                                   once its word has reached `epoch` (stands in for tile_signal /
+ *                                   tile_wait, sync/primitives.py:357-414, without consuming the flag)
  *   group_table int32[total_tiles]  S2: swizzled tile id -> group id (tile_group.py:214-241)
  *   counter    int32[n_groups]      S2: tile_signal_add / tile_wait_ge (tileccl_v2/ipc.py:231-254)
  *   barrier    int32[n_groups]      S2: finished communication tasks (or workgroups, see below) per group
  *   trace_*    optional device-clock stamps (signal.py:18-24); NULL to skip
  * locks, counter and barrier live in the symmetric heap, so a peer's copy sits at the
- * same offset in the peer's slice.  The host zeroes them before a launch
- * (TileGroupSignalState.reset, signal.py:32-40); `epoch` lets repeated launches reuse
- * unreset counters: a group is ready when counter[g] >= epoch * tile_counts[g]. */
+ * same offset in the peer's slice.  The host zeroes them once
+ * (TileGroupSignalState.reset, signal.py:32-40; wg_specialized.py:122-123 zeroes its locks per
+ * call); `epoch` lets repeated launches reuse them without a reset: a tile is ready when
+ * locks[t] >= epoch, a group when counter[g] >= epoch * tile_counts[g].  S1 and S2 launches
+ * on the same words number their launches separately (each counts the launches that wrote
+ * its words), and ranks that wait on each other must pass the same number. */
 typedef struct tccl_sync_desc {
   int32_t* locks;
   const int32_t* group_table;
   int32_t* counter;
   int32_t* barrier;
   int32_t n_groups;
-  int32_t epoch; /* >= 1 */
+  int32_t epoch; /* >= 1: the number of this launch among those of its variant on these words */
   const int32_t* row_starts; /* int32[n_groups], rows relative to the GEMM's C */
   const int32_t* row_ends;   /* clamped to M */
   const int32_t* tile_counts;

@@ -142,3 +142,28 @@ def test_cost_model_calibration_on_the_device(lib):
     finally:
         for h in heaps:
             h.cleanup()
+
+
+def test_tensors_outlive_the_heap_objects(lib):
+    """Heap objects cleaned up, dropped and garbage collected while a tensor allocated from
+    them is still held: the arena's device memory must stay until that tensor is gone."""
+    import gc
+    import weakref
+
+    from tileccl_amd.v2 import SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(1 << 20, 2)
+    arena = weakref.ref(heaps[0]._arena)
+    kept = heaps[1].allocate_tensor((64, 8), torch.float32)
+    kept.fill_(3.5)
+    for h in heaps:
+        h.cleanup()
+    del heaps, h
+    gc.collect()
+    assert arena() is not None and arena().live  # held by `kept` through its storage
+    assert torch.all(kept == 3.5).item()
+    with pytest.raises(RuntimeError, match="cleaned up"):
+        arena().slice(0)
+    del kept
+    gc.collect()
+    assert arena() is None  # collected, which is when the device memory is returned

@@ -143,16 +143,21 @@ def test_fp8_allgather_two_ranks(lib, variant, directions):
             h.cleanup()
 
 
-def test_baseline_config_4_properties(lib):
+@pytest.mark.parametrize("own_rows", [False, True])
+def test_baseline_config_4_properties(lib, own_rows):
     """16384x2048 @ 2048x4096 e4m3 with per-tensor scales, resident bf16 peer partial: the three
     variants agree byte for byte, the reduction equals the oracle on slabs of both owners, the
-    partial matches the dequantised matmul on a slab, counters match the plan."""
+    partial matches the dequantised matmul on a slab, counters match the plan; with the owned
+    rows kept in registers (what the benchmark runs) the outputs are the same bytes."""
+    from tests.test_gpu_reducescatter import check_full_size_config
     from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
 
     M, N, K = 16384, 4096, 2048
     heaps = SymmetricHeap.create_all(1 << 30, 2)
     try:
-        ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=torch.bfloat16, out_dtype=torch.bfloat16) for h in heaps]
+        kw = dict(partial_dtype=torch.bfloat16, out_dtype=torch.bfloat16)
+        ops = [FusedGemmReduceScatter(h, M, N, **kw) for h in heaps]
+        kept_ops = [FusedGemmReduceScatter(h, M, N, own_rows_in_registers=True, **kw) for h in heaps] if own_rows else None
         op = ops[0]
         assert op.plan.n_groups == 16 and op.shard_rows == 8192
         A_cpu, sa = quantise((M, K), 0)
@@ -160,24 +165,60 @@ def test_baseline_config_4_properties(lib):
         A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
         g = torch.Generator(device="cuda").manual_seed(2)
         ops[1].partial.copy_(torch.randn(M, N, generator=g, device="cuda").bfloat16())
-        outs = {}
-        for variant in ("s0", "s1", "s2"):
-            for o in ops:
-                o.out.zero_()
-            op.mark_peers_ready()
-            op(A, B, variant, scale_a=sa, scale_b=sb)
-            op.check_faults()
-            outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
-        for v in ("s1", "s2"):
-            assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
-        for owner in (0, 1):
-            rows = slice(owner * 8192 + 100, owner * 8192 + 228)
-            want = (op.partial[rows].float() + ops[1].partial[rows].float()).bfloat16()
-            assert torch.equal(bits(outs["s2"][owner][100:228]), bits(want))
-        rows = slice(8100, 8228)
-        ref = (A_cpu[rows].float() @ B_cpu.float()) * (sa * sb)
-        assert_gemm_close(op.partial[rows], ref, rtol=5e-2, tight=0.032)
-        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+
+        def gemm_ref(partial):
+            rows = slice(8100, 8228)
+            ref = (A_cpu[rows].float() @ B_cpu.float()) * (sa * sb)
+            assert_gemm_close(partial[rows], ref, rtol=5e-2, tight=0.032)
+
+        check_full_size_config(heaps, ops, kept_ops, A, B, 8192, torch.bfloat16, gemm_ref, 100, scale_a=sa, scale_b=sb)
     finally:
         for h in heaps:
             h.cleanup()
+
+
+@pytest.mark.parametrize("variant", ["s1", "s2"])
+@pytest.mark.parametrize("world,M", [(2, 1024), (3, 768)])
+def test_fp8_own_rows_kept_in_registers_give_the_same_bytes(lib, variant, world, M):
+    """fp8 inputs with the owned rows' partial kept in the accumulators: the fp8 kernels reduce
+    the other owners' rows by reading the stored partial back (a third code path next to the
+    two of the 16-bit kernels).  Outputs equal the oracle's reduction of the partials a plain
+    run stored, bit for bit (three ranks: order-sensitive magnitudes); the owned rows of
+    `partial` are never written, the other rows are."""
+    from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap
+
+    N, K = 528, 512  # e4m3 rows of B must be multiples of 16 bytes
+    A_cpu, sa = quantise((M, K), 0)
+    B_cpu, sb = quantise((K, N), 1, K**-0.5)
+    peers_cpu = {p: seeded((M, N), 10 + p, torch.bfloat16) * (1000.0 if world == 3 else 1.0) for p in range(1, world)}
+
+    def run(flag):
+        heaps = SymmetricHeap.create_all(64 << 20, world)
+        try:
+            ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=torch.bfloat16, out_dtype=torch.bfloat16,
+                                          tau_min_bytes=1, group_m=1, own_rows_in_registers=flag) for h in heaps]
+            A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+            for p in range(1, world):
+                ops[p].partial.copy_(peers_cpu[p])
+            for o in ops:
+                o.out.zero_()
+            ops[0].partial.fill_(-3.0)
+            ops[0].mark_peers_ready()
+            ops[0](A, B, variant, scale_a=sa, scale_b=sb)
+            ops[0].check_faults()
+            return ops[0].partial.cpu(), [o.out.cpu() for o in ops]
+        finally:
+            for h in heaps:
+                h.cleanup()
+
+    plain_partial, plain_outs = run(False)
+    kept_partial, kept_outs = run(True)
+    assert_gemm_close(plain_partial, (A_cpu.float() @ B_cpu.float()) * (sa * sb), rtol=5e-2, tight=0.032)
+    shard = M // world
+    partials = [plain_partial] + [peers_cpu[p] for p in range(1, world)]
+    for owner in range(world):
+        want = oracle.reduce_rows(partials, owner, torch.bfloat16)
+        assert torch.equal(bits(plain_outs[owner]), bits(want)), owner
+        assert torch.equal(bits(kept_outs[owner]), bits(want)), owner
+    assert torch.all(kept_partial[:shard] == -3.0)  # never stored
+    assert torch.equal(bits(kept_partial[shard:]), bits(plain_partial[shard:]))

@@ -146,34 +146,67 @@ def test_own_rows_kept_in_registers_give_the_same_bytes(lib, variant, world, M, 
     assert torch.equal(bits(kept_partial[shard:]), bits(plain_partial[shard:]))
 
 
-def test_baseline_config_3_properties(lib):
+def check_full_size_config(heaps, ops, kept_ops, A, B, shard, out_dtype, gemm_ref, slab_lo, **scales):
+    """Shared body of the full-size reduce-scatter configurations.  `ops` store every partial;
+    `kept_ops` (or None) are the same operation with the owned rows' partial kept in the
+    accumulators, which is the mode the benchmark times."""
+    op = ops[0]
+    outs = {}
+    for variant in VARIANTS:
+        for o in ops:
+            o.out.zero_()
+        op.mark_peers_ready()
+        op(A, B, variant, **scales)
+        op.check_faults()
+        outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
+    for v in ("s1", "s2"):
+        assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
+    for owner in (0, 1):
+        rows = slice(owner * shard + slab_lo, owner * shard + slab_lo + 128)
+        want = (op.partial[rows].float() + ops[1].partial[rows].float()).to(out_dtype)
+        assert torch.equal(bits(outs["s2"][owner][slab_lo:slab_lo + 128]), bits(want))
+    gemm_ref(op.partial)
+    assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+    if kept_ops is None:
+        return
+    kept = kept_ops[0]
+    kept_ops[1].partial.copy_(ops[1].partial)
+    for variant in ("s1", "s2"):
+        for o in kept_ops:
+            o.out.zero_()
+        kept.partial.fill_(-3.0)
+        kept.mark_peers_ready()
+        kept(A, B, variant, **scales)
+        kept.check_faults()
+        for owner in (0, 1):  # the bytes of the bulk variant on stored partials
+            assert torch.equal(bits(kept_ops[owner].out), bits(outs["s0"][owner])), (variant, owner)
+        assert torch.all(kept.partial[:shard] == -3.0), variant  # the owned rows' partial is never stored
+        assert torch.equal(bits(kept.partial[shard:]), bits(op.partial[shard:])), variant
+    assert kept.signals.counter.tolist() == oracle.expected_counters(kept.plan.tile_counts(), kept.words.epoch)
+
+
+@pytest.mark.parametrize("own_rows", [False, True])
+def test_baseline_config_3_properties(lib, own_rows):
     """8192x2048 @ 2048x4096 fp16, peer partial fp32 N(0,1): variants agree byte for byte,
-    the result equals the oracle on a slab, counters match the plan."""
+    the result equals the oracle on a slab, counters match the plan; with the owned rows kept
+    in registers (what the benchmark runs) the outputs are the same bytes."""
+    from tileccl_amd.v2 import FusedGemmReduceScatter
+
     M, N, K = 8192, 4096, 2048
     heaps, ops = make(2, M, N, heap_bytes=1 << 30)
     try:
         op = ops[0]
         assert op.plan.n_groups == 8 and op.shard_rows == 4096
+        kept_ops = [FusedGemmReduceScatter(h, M, N, own_rows_in_registers=True) for h in heaps] if own_rows else None
         A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=K**-0.5))
         g = torch.Generator(device="cuda").manual_seed(2)
         ops[1].partial.normal_(generator=g)
-        outs = {}
-        for variant in VARIANTS:
-            for o in ops:
-                o.out.zero_()
-            op.mark_peers_ready()
-            op(A, B, variant)
-            op.check_faults()
-            outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
-        for v in ("s1", "s2"):
-            assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
-        for owner in (0, 1):
-            rows = slice(owner * 4096, owner * 4096 + 128)
-            want = (op.partial[rows].float() + ops[1].partial[rows].float()).half()
-            assert torch.equal(bits(outs["s2"][owner][:128]), bits(want))
-        rows = slice(4000, 4128)
-        assert_gemm_close(op.partial[rows], A[rows].float().cpu() @ B.float().cpu(), tight=1e-3)
-        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+
+        def gemm_ref(partial):
+            rows = slice(4000, 4128)
+            assert_gemm_close(partial[rows], A[rows].float().cpu() @ B.float().cpu(), tight=1e-3)
+
+        check_full_size_config(heaps, ops, kept_ops, A, B, 4096, torch.float16, gemm_ref, 0)
     finally:
         for h in heaps:
             h.cleanup()

@@ -95,3 +95,55 @@ def test_context_shape_normalisation_and_missing_heap():
     with pytest.raises(RuntimeError, match="has not been initialised"):
         tileccl_amd._ctx = None
         tileccl_amd.current_context()
+
+
+class _FakeArena:
+    """The arena's bookkeeping over host memory: the three device hooks are replaced."""
+
+    freed: list = []
+
+    def __new__(cls, *args, **kwargs):
+        from tileccl_amd.memory.arena import Arena
+
+        class Fake(Arena):
+            def _allocate(self, slice_bytes, world_size):
+                return ("handle", slice_bytes), [4096 + r * slice_bytes for r in range(world_size)]
+
+            def _view(self, base, nbytes):
+                return torch.zeros(nbytes, dtype=torch.uint8)
+
+            def _device_bases(self, bases):
+                return torch.tensor(bases, dtype=torch.int64)
+
+            def _deallocate(self, handle):
+                _FakeArena.freed.append(handle)
+
+        return Fake(*args, **kwargs)
+
+
+def test_arena_is_freed_when_collected_not_when_the_last_heap_lets_go():
+    import gc
+
+    _FakeArena.freed = []
+    arena = _FakeArena(1024, 2)
+    users = [arena.acquire(), arena.acquire()]
+    assert arena.live and arena.slice(1).numel() == 1024
+    users[0].release()
+    assert arena.live and arena.slice(0) is not None  # one heap still uses it
+    users[1].release()
+    assert arena.live and _FakeArena.freed == []  # nothing is freed under tensors that may still view it
+    with pytest.raises(RuntimeError, match="cleaned up"):
+        arena.slice(0)
+    assert arena.heap_bases is None
+    del arena, users
+    gc.collect()
+    assert _FakeArena.freed == [("handle", 1024)]  # exactly once, when nothing refers to the arena
+
+
+def test_arena_rejects_bad_sizes_before_allocating():
+    _FakeArena.freed = []
+    with pytest.raises(ValueError, match="Heap size must be positive"):
+        _FakeArena(0, 1)
+    with pytest.raises(ValueError, match="world_size must be >= 1"):
+        _FakeArena(16, 0)
+    assert _FakeArena.freed == []

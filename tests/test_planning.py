@@ -145,6 +145,9 @@ def test_plan_with_owner_split():
     # groups before the split: waves of 16 tiles -> [(0,1024,16),(1024,2048,16)]; cut at 512
     assert plan.groups == [(0, 512, 8), (512, 1024, 8), (1024, 2048, 16)]
     assert plan.group_table.tolist() == ref.group_table(2048, 256, plan.groups)
+    # None means "no boundaries" (reference tile_group.py:269), the same as an empty sequence
+    assert build_tile_group_plan(2048, 256, FP16_TILE, row_split_boundaries=None).groups == \
+        build_tile_group_plan(2048, 256, FP16_TILE).groups == [(0, 1024, 16), (1024, 2048, 16)]
 
 
 # ---- validation ------------------------------------------------------------------------------------

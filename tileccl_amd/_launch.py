@@ -133,10 +133,14 @@ class DevicePlan:
 class SyncWords:
     """Signal words of one fused operation plus the launch epoch.
 
-    Counters grow monotonically: launch ``e`` (1-based) treats group ``g`` as ready at
-    ``counter[g] >= e * tile_counts[g]``, so repeated launches need no reset kernel.
-    ``reset()`` zeroes the words and restarts the epoch, which is also what happens
-    automatically before the 32-bit counters could overflow.
+    Counters grow monotonically: TileGroup launch ``e`` (1-based) treats group ``g`` as ready
+    at ``counter[g] >= e * tile_counts[g]``, and tile-by-tile launch ``e`` stores ``e`` into
+    ``locks[tile]`` and treats a tile as ready at ``locks[tile] >= e``, so repeated launches
+    need no reset kernel and a flag of an earlier launch is never mistaken for this one's.
+    The two kinds of launch count separately (``epoch`` / ``lock_epoch``): each numbers the
+    launches that wrote its own words.  Ranks that wait on each other's words must have issued
+    the same number of launches.  ``reset()`` zeroes the words and restarts both numbers,
+    which is also what happens automatically before the 32-bit words could overflow.
 
     A launch recorded into a HIP graph replays with the arguments it was recorded with, so
     its epoch cannot advance.  A TileGroup launch issued while the stream is capturing is
@@ -156,6 +160,7 @@ class SyncWords:
     trace_done_clock: torch.Tensor | None = None
     fault: torch.Tensor = field(default_factory=lambda: torch.zeros(1, dtype=torch.int64, device="cuda:0"))
     epoch: int = 0
+    lock_epoch: int = 0
     spin_limit_ns: int = DEFAULT_SPIN_LIMIT_NS
     max_tasks_per_tile: int = 1 << 16
     clear_every_launch: bool = False  # set by the first launch recorded into a graph
@@ -166,22 +171,27 @@ class SyncWords:
             if t is not None:
                 t.zero_()
         self.epoch = 0
+        self.lock_epoch = 0
 
-    def next_epoch(self) -> int:
+    def next_epoch(self, variant: str = "s2") -> int:
+        """Number the launch about to be issued: ``"s2"`` advances ``epoch``, ``"s1"`` ``lock_epoch``."""
+        tile_by_tile = variant == "s1"
         if self.clear_every_launch or torch.cuda.is_current_stream_capturing():
             self.clear_every_launch = True
-            for t in (self.counter, self.barrier):
+            for t in (self.locks, self.counter, self.barrier):
                 if t is not None:
                     t.zero_()
-            self.epoch = 1
-            return 1
-        if self.epoch >= (1 << 30) // self.max_tasks_per_tile:
+            self.epoch = self.lock_epoch = 0
+        elif max(self.epoch, self.lock_epoch) >= (1 << 30) // self.max_tasks_per_tile:
             torch.cuda.current_stream().synchronize()
             self.reset()
+        if tile_by_tile:
+            self.lock_epoch += 1
+            return self.lock_epoch
         self.epoch += 1
         return self.epoch
 
-    def desc(self) -> _lib.SyncDesc:
+    def desc(self, variant: str = "s2") -> _lib.SyncDesc:
         s = _lib.SyncDesc()
         s.locks = ptr(self.locks)
         s.counter = ptr(self.counter)
@@ -192,7 +202,7 @@ class SyncWords:
             s.row_ends = ptr(self.plan.row_ends)
             s.tile_counts = ptr(self.plan.tile_counts)
             s.n_groups = self.plan.n_groups
-        s.epoch = max(self.epoch, 1)
+        s.epoch = max(self.lock_epoch if variant == "s1" else self.epoch, 1)
         s.trace_comm_counter = ptr(self.trace_comm_counter)
         s.trace_start_clock = ptr(self.trace_start_clock)
         s.trace_ready_clock = ptr(self.trace_ready_clock)

@@ -297,10 +297,10 @@ int check_sync(const tccl_sync_desc* s, int variant) {
   if (variant == TCCL_S0_BULK) return 0;
   if (!s) return fail(TCCL_ERR_INVALID, "variant S%d needs a sync descriptor", variant);
   if (variant == TCCL_S1_TILE && !s->locks) return fail(TCCL_ERR_INVALID, "S1 needs locks");
+  if (s->epoch < 1) return fail(TCCL_ERR_INVALID, "S%d epoch must be >= 1", variant);
   if (variant == TCCL_S2_TILEGROUP) {
     if (!s->counter || !s->group_table || !s->row_starts || !s->row_ends || !s->tile_counts || s->n_groups <= 0)
       return fail(TCCL_ERR_INVALID, "S2 needs counter, group_table, row_starts, row_ends, tile_counts and n_groups > 0");
-    if (s->epoch < 1) return fail(TCCL_ERR_INVALID, "S2 epoch must be >= 1");
   }
   return 0;
 }
@@ -544,6 +544,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     f.g = g;
     f.m = m;
     f.trace_start = trace_start;
+    s.epoch = sync->epoch > 0 ? sync->epoch : 1;
     if (variant == TCCL_S1_TILE) {
       s.mode = tccl::kSignalTile;
       s.locks = sync->locks;
@@ -553,7 +554,6 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
       s.counter = sync->counter;
       s.group_table = sync->group_table;
       s.tile_counts = sync->tile_counts;
-      s.epoch = sync->epoch > 0 ? sync->epoch : 1;
       s.trace_ready_clock = sync->trace_ready_clock;
       c.granularity = tccl::kPerGroup;
     }
@@ -582,6 +582,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     return launch_comm(c, bulk_comm_wgs(dev), stream);
   }
   int comm = tr && tr->num_comm_wgs > 0 ? tr->num_comm_wgs : dev.compute_units;
+  s.epoch = sync->epoch > 0 ? sync->epoch : 1;
   if (variant == TCCL_S1_TILE) {
     s.mode = tccl::kSignalTile;
     s.locks = sync->locks;

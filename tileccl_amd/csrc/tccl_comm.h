@@ -16,7 +16,7 @@
 //   gather-columns  rank p's input shard -> column block p of this rank's gathered input
 //                   [gather worker of patterns/chained_ag_gemm_rs.py:262-340]
 // and three granularities: bulk (no waiting; the second kernel of S0), per plan tile
-// (S1: tile_wait on locks[tile]) and per TileGroup (S2: tile_wait_ge on counter[group]).
+// (S1: locks[tile] >= epoch) and per TileGroup (S2: tile_wait_ge on counter[group]).
 #pragma once
 
 #include "tccl_device.h"
@@ -384,13 +384,13 @@ struct Waiter {
     return all_ok;  // the data itself is read with device-coherent loads: no cache invalidate
   }
 
-  // S1: locks[tile] of `rank`'s slice.  Own locks are consumed (tile_wait); a peer's are
-  // only observed (tile_poll), since the peer's own workgroups consume them.
+  // S1: locks[tile] of `rank`'s slice has reached this launch's epoch (tile_publish).  The
+  // word is only observed, whoever owns it: several parties may depend on the same tile.
   TCCL_D bool tile(int tile_id, int rank) const {
     bool ok = true;
     if (threadIdx.x == 0) {
-      int32_t* w = translate_ptr(a.locks, a.rank, rank, a.heap_bases);
-      ok = tile_wait<true>(w, tile_id, /*consume=*/rank == a.rank, deadline);
+      const int32_t* w = translate_ptr(a.locks, a.rank, rank, a.heap_bases);
+      ok = tile_wait_ge<true>(w, tile_id, a.epoch, deadline);
     }
     return finish(ok);
   }

@@ -132,6 +132,16 @@ TCCL_D bool tile_wait(int32_t* locks, int i, bool consume, int64_t deadline) {
   }
 }
 
+// Epoch-valued tile flags of the fused tile-by-tile launches: launch e stores e into
+// locks[tile], and a tile counts as ready for launch e once its word has reached e
+// (tile_wait_ge).  Nothing is consumed, so the owner's communication role and any number of
+// peers can watch the same word, and a flag left behind by launch e-1 is never taken for
+// launch e's.  (The reference gets the second property by zeroing its lock tensor before
+// every call: patterns/wg_specialized.py:122-123.)
+TCCL_D void tile_publish(int32_t* locks, int i, int32_t epoch) {
+  __hip_atomic_store(&locks[i], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // tile_signal_add: counter[i] += v; returns the previous value. (ipc.py:231-241)
 template <bool Relaxed = false>
 TCCL_D int32_t tile_signal_add(int32_t* words, int i, int32_t v) {

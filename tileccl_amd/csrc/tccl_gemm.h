@@ -61,9 +61,9 @@ struct SignalArgs {
   int32_t* locks;
   const int32_t* group_table;
   int32_t* counter;
-  // optional device trace: the producer that completes a group stamps its clock
   const int32_t* tile_counts;
-  int epoch;
+  int epoch;  // launch number: locks[tile] = epoch (tile mode); a group is complete at epoch * tile_counts[g]
+  // optional device trace: the producer that completes a group stamps its clock
   int64_t* trace_ready_clock;
 };
 
@@ -304,7 +304,7 @@ struct GemmRole {
         __syncthreads();
         if (tid == 0) {
           if (s.mode == kSignalTile)
-            tile_signal<true>(s.locks, tile_id);
+            tile_publish(s.locks, tile_id, s.epoch);
           else
             tile_signal_add<true>(s.counter, s.group_table[tile_id], 1);
         }

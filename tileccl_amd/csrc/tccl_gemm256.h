@@ -1127,7 +1127,7 @@ struct Gemm256 {
             if (tm >= g.tile_rows || tn >= g.tile_cols) continue;
             const int tile_id = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
             if (s.mode == kSignalTile) {
-              ok = tile_wait<true>((int32_t*)((char*)ra->locks + delta), tile_id, /*consume=*/false, deadline);
+              ok = tile_wait_ge<true>((const int32_t*)((const char*)ra->locks + delta), tile_id, ra->epoch, deadline);
             } else {
               const int gi = s.group_table[tile_id];
               if (gi == waited_group) continue;
@@ -1231,7 +1231,7 @@ struct Gemm256 {
         if (tm >= g.tile_rows || tn >= g.tile_cols) continue;
         const int tile_id = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
         if (s.mode == kSignalTile) {
-          tile_signal<true>(s.locks, tile_id);
+          tile_publish(s.locks, tile_id, s.epoch);
           continue;
         }
         const int gi = s.group_table[tile_id];

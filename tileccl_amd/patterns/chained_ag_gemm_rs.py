@@ -113,8 +113,9 @@ class ChainedAGGemmRSPattern:
         words = self._stage._sync_words(M, N, output)
         sync = None
         if words is not None:
-            words.next_epoch()
-            sync = words.desc()
+            variant = "s1" if self._stage.variant == _lib.S1_TILE else "s2"
+            words.next_epoch(variant)
+            sync = words.desc(variant)
         rc = _lib.load().tccl_chained_ag_gemm_rs(
             C.byref(gemm),
             _launch.ptr(input_shard),

@@ -81,8 +81,9 @@ class _HipAllScatterPattern(Pattern):
         words = self._sync_words(spec.M, spec.local_N, C_out)
         sync = None
         if words is not None:
-            words.next_epoch()
-            sync = words.desc()
+            variant = "s1" if self.variant == _lib.S1_TILE else "s2"
+            words.next_epoch(variant)
+            sync = words.desc(variant)
         rc = _lib.load().tccl_gemm_allscatter(
             C.byref(gemm),
             C.byref(scatter),

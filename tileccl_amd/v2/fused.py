@@ -30,7 +30,7 @@ from tileccl_amd.v2.signal import TileGroupSignalState, allocate_tile_group_sign
 from tileccl_amd.v2.tile_group import TileGroupPlan, build_tile_group_plan
 from tileccl_amd.v2.transport import CommMode, P2PTransportPlan, build_p2p_transport_plan
 
-PEER_READY = 1 << 30  # counter value that marks a resident peer's groups as complete
+PEER_READY = 1 << 30  # word value that marks a resident peer's tiles / groups as complete for every launch
 
 
 def _directions(value) -> int:
@@ -135,7 +135,7 @@ class _FusedBase:
             if peer == self.rank:
                 continue
             self.heap.peer_view(self.signals.counter, peer).fill_(PEER_READY)
-            self.heap.peer_view(self.locks, peer).fill_(1)
+            self.heap.peer_view(self.locks, peer).fill_(PEER_READY)
 
     def _descs(self, directions: int, variant: str):
         assert self.words is not None
@@ -145,9 +145,9 @@ class _FusedBase:
         transport = _launch.transport_desc(
             directions, self.transport.copy_elems, self.transport.reduce_elems, self.num_comm_wgs
         )
-        if variant == "s2":  # only S2 launches add to the counters, so only they advance the epoch
-            self.words.next_epoch()
-        return view, transport, self.words.desc()
+        if variant != "s0":  # S1 launches number the locks they write, S2 launches the counters
+            self.words.next_epoch(variant)
+        return view, transport, self.words.desc(variant)
 
     def check_faults(self) -> None:
         if self.words is not None:

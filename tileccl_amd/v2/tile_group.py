@@ -277,7 +277,7 @@ def build_tile_group_plan(
     block_n: int = DEFAULT_BLOCK_N,
     group_m: int = DEFAULT_GROUP_M,
     tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES,
-    row_split_boundaries: Iterable[int] = (),
+    row_split_boundaries: Iterable[int] | None = (),
 ) -> TileGroupPlan:
     """Groups (optionally cut at owner boundaries) plus their swizzle table, as one plan."""
     groups = build_tile_groups(
@@ -291,7 +291,7 @@ def build_tile_group_plan(
         group_m=group_m,
         tau_min_bytes=tau_min_bytes,
     )
-    cuts = list(row_split_boundaries)
+    cuts = list(row_split_boundaries or ())  # None: no boundaries, as the reference accepts (tile_group.py:269)
     if cuts:
         groups = split_groups_at_row_boundaries(M, N, groups, cuts, block_m=block_m, block_n=block_n)
     return TileGroupPlan(
