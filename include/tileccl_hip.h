@@ -284,6 +284,43 @@ int tccl_gemm_reducescatter(const tccl_gemm_desc* gemm, void* out, int32_t out_d
                             const tccl_transport_desc* transport, int32_t emulate_peer,
                             int32_t variant, void* stream);
 
+/* ---- one entry point that allocates nothing ------------------------------------------------
+ * No counterpart in the reference (its lock / signal tensors are torch allocations made by
+ * the caller's process: wg_specialized.py:104-124, tileccl_v2/signal.py:43-66).  It is for
+ * callers that cannot allocate device memory for the signal words: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.
+ *
+ * tccl_gemm_allgather (S1 or S2) with the signal words and plan tables -- locks, counter,
+ * barrier, group_table, row_starts, row_ends, tile_counts -- kept in a file-scope device array
+ * of the library (about 581 KiB on every GPU the process uses, for the life of the process)
+ * instead of being brought in by a tccl_sync_desc.  The caller still passes the operands, the
+ * gathered output and the heap view; `plan` is HOST memory and travels in the kernel
+ * arguments of a small set-up kernel that also clears the calling rank's words, so every call
+ * runs as launch number 1.  group_table is derived on the device from the plan's rows by the
+ * rule of build_group_table (tileccl_v2/tile_group.py:214-241).
+ *
+ * Limits: at most TCCL_STATIC_MAX_TILES plan tiles and TCCL_STATIC_MAX_GROUPS TileGroups
+ * (larger inputs are rejected with TCCL_ERR_UNSUPPORTED), groups ascending and disjoint.
+ * The ranks emulated on one GPU share the array, each with its own block of words: a rank
+ * that pulls finds a peer's words where that peer's own last call left them.  Calls that
+ * overlap in time on one GPU race on the shared plan tables (and on their own words when
+ * they are calls of the same rank): order them on one stream.  The first call on a device
+ * looks up the array's address (no allocation); make it before a capture begins.
+ * `fault` (device int64[1] or NULL) and `spin_limit_ns` as in tccl_sync_desc.  Calls
+ * no hipMalloc / hipFree and no allocating library routine. */
+#define TCCL_STATIC_MAX_TILES 16384
+#define TCCL_STATIC_MAX_GROUPS 64
+typedef struct tccl_static_plan {
+  int32_t n_groups; /* 1 .. TCCL_STATIC_MAX_GROUPS */
+  int32_t row_starts[TCCL_STATIC_MAX_GROUPS]; /* rows relative to the GEMM's C */
+  int32_t row_ends[TCCL_STATIC_MAX_GROUPS];   /* clamped to M */
+  int32_t tile_counts[TCCL_STATIC_MAX_GROUPS];
+} tccl_static_plan;
+int tccl_gemm_allgather_static(const tccl_gemm_desc* gemm, void* out, int64_t ld_out,
+                               const tccl_heap_view* heap, const tccl_static_plan* plan,
+                               const tccl_transport_desc* transport, int32_t variant,
+                               int64_t* fault, int64_t spin_limit_ns, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

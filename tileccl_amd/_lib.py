@@ -105,6 +105,20 @@ class TransportDesc(C.Structure):
     ]
 
 
+STATIC_MAX_TILES, STATIC_MAX_GROUPS = 16384, 64
+
+
+class StaticPlan(C.Structure):
+    """Host-side plan rows of ``tccl_gemm_allgather_static`` (``tccl_static_plan``)."""
+
+    _fields_ = [
+        ("n_groups", C.c_int32),
+        ("row_starts", C.c_int32 * STATIC_MAX_GROUPS),
+        ("row_ends", C.c_int32 * STATIC_MAX_GROUPS),
+        ("tile_counts", C.c_int32 * STATIC_MAX_GROUPS),
+    ]
+
+
 _P = C.POINTER
 _i32, _i64, _vp = C.c_int32, C.c_int64, C.c_void_p
 
@@ -142,6 +156,10 @@ SIGNATURES = {
     "tccl_gemm_allgather": (
         C.c_int,
         [_P(GemmDesc), _vp, _i64, _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],
+    ),
+    "tccl_gemm_allgather_static": (
+        C.c_int,
+        [_P(GemmDesc), _vp, _i64, _P(HeapView), _P(StaticPlan), _P(TransportDesc), _i32, _vp, _i64, _vp],
     ),
     "tccl_gemm_reducescatter": (
         C.c_int,

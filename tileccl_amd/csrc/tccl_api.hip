@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/tileccl_hip.h"
 #include "tccl_comm.h"
@@ -438,6 +439,7 @@ bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   p->trace_done_clock = c.trace_done_clock;
   p->fault = c.fault;
   p->spin_ticks = c.spin_ticks;
+  p->word_stride = c.word_stride;
   return true;
 }
 
@@ -594,6 +596,103 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     c.granularity = tccl::kPerGroup;
   }
   return launch_fused(d->in_dtype, d->out_dtype, g, s, c, compute, comm, trace_start, stream);
+}
+
+
+// GEMM-output AllGather.  word_stride: 0 when the ranks' signal words live in the heap (a
+// peer's at the same slice offset), else the distance between consecutive ranks' words.
+int allgather_impl(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap, const tccl_sync_desc* sync,
+                   const tccl_transport_desc* tr, int32_t variant, int64_t word_stride, hipStream_t stream) {
+  int rc = check_gemm(d);
+  if (rc) return rc;
+  if ((rc = check_heap(heap))) return rc;
+  if (variant < TCCL_S0_BULK || variant > TCCL_S2_TILEGROUP) return fail(TCCL_ERR_INVALID, "unknown variant %d", variant);
+  if ((rc = check_sync(sync, variant))) return rc;
+  if (!out) return fail(TCCL_ERR_INVALID, "allgather: out is NULL");
+  const int esize = (int)dtype_size(d->out_dtype);
+  if (ld_out != d->ldc) return fail(TCCL_ERR_INVALID, "allgather: ld_out must equal the GEMM's ldc");
+  const char* want = (const char*)out + (int64_t)heap->rank * d->M * ld_out * esize;
+  if ((const char*)d->C != want) return fail(TCCL_ERR_INVALID, "allgather: gemm C must point at row rank*M of out");
+  if ((d->N * esize) % 16 || (ld_out * esize) % 16) return fail(TCCL_ERR_UNSUPPORTED, "allgather: rows must be multiples of 16 bytes");
+  if (tr && !(tr->directions & (TCCL_DIR_PUSH | TCCL_DIR_PULL))) return fail(TCCL_ERR_INVALID, "allgather: no transfer direction selected");
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  tccl::GemmArgs g;
+  build_gemm_args(d, dev, &g);
+  tccl::CommArgs c;
+  fill_comm_common(&c, g, esize, heap, sync, tr);
+  c.op = tccl::kOpAllGather;
+  c.out = (char*)out;
+  c.ld_out_bytes = ld_out * esize;
+  c.word_stride = word_stride;
+  if ((rc = set_task_units(&c, tr, false))) return rc;
+  return run_variant(d, c, sync, tr, variant, dev, g, stream);
+}
+
+// ---- signal words that the library keeps itself (tccl_gemm_allgather_static) --------------------
+// One rank's words, then the next rank's: a peer's words are a fixed distance away.
+struct StaticWords {
+  int32_t locks[TCCL_STATIC_MAX_TILES];
+  int32_t counter[TCCL_STATIC_MAX_GROUPS];
+  int32_t barrier[TCCL_STATIC_MAX_GROUPS];
+};
+struct StaticScratch {
+  int32_t group_table[TCCL_STATIC_MAX_TILES];
+  int32_t row_starts[TCCL_STATIC_MAX_GROUPS];
+  int32_t row_ends[TCCL_STATIC_MAX_GROUPS];
+  int32_t tile_counts[TCCL_STATIC_MAX_GROUPS];
+  StaticWords words[TCCL_MAX_WORLD];
+};
+// Device memory that exists from the moment the library is loaded: about 581 KiB on every
+// GPU the process uses.  In host code this name is only a handle for hipGetSymbolAddress; the
+// address kernels and copies may use is the one static_scratch() returns.
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratch)];
+
+constexpr int kMaxDevices = 64;
+StaticScratch* g_scratch_ptr[kMaxDevices];  // per device, resolved on first use
+std::mutex g_scratch_mutex;
+
+// The current device's copy of the scratch.  The first call on a device asks the runtime for
+// the symbol's address on that device (no allocation); later calls read the cached pointer.
+int static_scratch(StaticScratch** out) {
+  int device = -1;
+  TCCL_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(TCCL_ERR_NO_DEVICE, "device %d outside [0, %d)", device, kMaxDevices);
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    TCCL_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(TCCL_ERR_NO_DEVICE, "the static scratch has no address on device %d", device);
+    g_scratch_ptr[device] = (StaticScratch*)p;
+  }
+  *out = g_scratch_ptr[device];
+  return 0;
+}
+
+// Clears rank `rank`'s words and writes the plan tables: group_table by the rule of
+// build_group_table (tileccl_v2/tile_group.py:214-241: the first group whose rows contain the
+// tile's first row, 0 if none), under the tile numbering of tile_coords.  The other ranks'
+// words are left as their own last call left them.
+__global__ void static_setup_kernel(StaticScratch* s, tccl_static_plan plan, int rank, int tile_rows, int tile_cols, int block_m,
+                                    int group_m) {
+  const int total = tile_rows * tile_cols;
+  StaticWords* mine = &s->words[rank];
+  const int first = blockIdx.x * blockDim.x + threadIdx.x, stride = gridDim.x * blockDim.x;
+  for (int t = first; t < total; t += stride) {
+    const int row = tccl::tile_coords(t, tile_rows, tile_cols, group_m).m * block_m;
+    int gid = 0;
+    for (int g = plan.n_groups - 1; g >= 0; --g)
+      if (plan.row_starts[g] <= row && row < plan.row_ends[g]) gid = g;
+    s->group_table[t] = gid;
+    mine->locks[t] = 0;
+  }
+  for (int g = first; g < plan.n_groups; g += stride) {
+    s->row_starts[g] = plan.row_starts[g];
+    s->row_ends[g] = plan.row_ends[g];
+    s->tile_counts[g] = plan.tile_counts[g];
+    mine->counter[g] = 0;
+    mine->barrier[g] = 0;
+  }
 }
 
 }  // namespace
@@ -971,29 +1070,54 @@ int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* d, const void* shard, int64_t 
 
 int tccl_gemm_allgather(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap,
                         const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, void* stream) {
+  return allgather_impl(d, out, ld_out, heap, sync, tr, variant, 0, (hipStream_t)stream);
+}
+
+int tccl_gemm_allgather_static(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap,
+                               const tccl_static_plan* plan, const tccl_transport_desc* tr, int32_t variant,
+                               int64_t* fault, int64_t spin_limit_ns, void* stream) {
   int rc = check_gemm(d);
   if (rc) return rc;
   if ((rc = check_heap(heap))) return rc;
-  if (variant < TCCL_S0_BULK || variant > TCCL_S2_TILEGROUP) return fail(TCCL_ERR_INVALID, "unknown variant %d", variant);
-  if ((rc = check_sync(sync, variant))) return rc;
-  if (!out) return fail(TCCL_ERR_INVALID, "allgather: out is NULL");
-  const int esize = (int)dtype_size(d->out_dtype);
-  if (ld_out != d->ldc) return fail(TCCL_ERR_INVALID, "allgather: ld_out must equal the GEMM's ldc");
-  const char* want = (const char*)out + (int64_t)heap->rank * d->M * ld_out * esize;
-  if ((const char*)d->C != want) return fail(TCCL_ERR_INVALID, "allgather: gemm C must point at row rank*M of out");
-  if ((d->N * esize) % 16 || (ld_out * esize) % 16) return fail(TCCL_ERR_UNSUPPORTED, "allgather: rows must be multiples of 16 bytes");
-  if (tr && !(tr->directions & (TCCL_DIR_PUSH | TCCL_DIR_PULL))) return fail(TCCL_ERR_INVALID, "allgather: no transfer direction selected");
-  tccl_device_info dev;
-  if ((rc = query_device(-1, &dev))) return rc;
-  tccl::GemmArgs g;
-  build_gemm_args(d, dev, &g);
-  tccl::CommArgs c;
-  fill_comm_common(&c, g, esize, heap, sync, tr);
-  c.op = tccl::kOpAllGather;
-  c.out = (char*)out;
-  c.ld_out_bytes = ld_out * esize;
-  if ((rc = set_task_units(&c, tr, false))) return rc;
-  return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+  if (variant != TCCL_S1_TILE && variant != TCCL_S2_TILEGROUP)
+    return fail(TCCL_ERR_INVALID, "allgather_static: variant %d keeps no signal words; use tccl_gemm_allgather with sync = NULL", variant);
+  if (!plan) return fail(TCCL_ERR_INVALID, "allgather_static: plan is NULL");
+  if (plan->n_groups < 1 || plan->n_groups > TCCL_STATIC_MAX_GROUPS)
+    return fail(TCCL_ERR_INVALID, "allgather_static: n_groups=%d outside [1, %d]", plan->n_groups, TCCL_STATIC_MAX_GROUPS);
+  const int tile_rows = (d->M + d->block_m - 1) / d->block_m, tile_cols = (d->N + d->block_n - 1) / d->block_n;
+  const int64_t tiles = (int64_t)tile_rows * tile_cols;
+  if (tiles > TCCL_STATIC_MAX_TILES)
+    return fail(TCCL_ERR_UNSUPPORTED, "allgather_static: %lld plan tiles exceed the static scratch (%d tiles)", (long long)tiles, TCCL_STATIC_MAX_TILES);
+  for (int g = 0; g < plan->n_groups; ++g)
+    if (plan->row_starts[g] < 0 || plan->row_ends[g] <= plan->row_starts[g] || plan->row_ends[g] > d->M || plan->tile_counts[g] <= 0 ||
+        (g > 0 && plan->row_starts[g] < plan->row_ends[g - 1]))
+      return fail(TCCL_ERR_INVALID, "allgather_static: group %d = rows [%d, %d), %d tiles is not an ascending cover of M=%d", g,
+                  plan->row_starts[g], plan->row_ends[g], plan->tile_counts[g], d->M);
+  StaticScratch* sc = nullptr;
+  if ((rc = static_scratch(&sc))) return rc;
+  // One small kernel clears this rank's words and (re)writes the plan tables; it is ordered
+  // before the fused launch by the stream.  Nothing is allocated and nothing is memset.
+  const int threads = 256;
+  int blocks = (int)((tiles + threads - 1) / threads);
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(static_setup_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, sc, *plan, heap->rank, tile_rows, tile_cols,
+                     d->block_m, d->group_m);
+  TCCL_HIP(hipGetLastError());
+  tccl_sync_desc sync;
+  memset(&sync, 0, sizeof sync);
+  StaticWords* mine = &sc->words[heap->rank];
+  sync.locks = mine->locks;
+  sync.counter = mine->counter;
+  sync.barrier = mine->barrier;
+  sync.group_table = sc->group_table;
+  sync.row_starts = sc->row_starts;
+  sync.row_ends = sc->row_ends;
+  sync.tile_counts = sc->tile_counts;
+  sync.n_groups = plan->n_groups;
+  sync.epoch = 1;
+  sync.fault = fault;
+  sync.spin_limit_ns = spin_limit_ns;
+  return allgather_impl(d, out, ld_out, heap, &sync, tr, variant, (int64_t)sizeof(StaticWords), (hipStream_t)stream);
 }
 
 int tccl_gemm_reducescatter(const tccl_gemm_desc* d, void* out, int32_t out_dtype, int64_t ld_out,

@@ -71,7 +71,18 @@ struct CommArgs {
   int64_t* fault;
   int64_t spin_ticks;
   int copy_units, reduce_units;  // units per task
+  // Where a peer's signal words are.  0: in the peer's heap slice, at the offset of this
+  // rank's.  Otherwise the ranks' words are consecutive blocks of this many bytes outside the
+  // heap, rank r's block starting (r - rank) * word_stride bytes from this rank's.
+  int64_t word_stride;
 };
+
+// Rank `rank`'s copy of the signal words `own` of rank a.rank.
+template <typename T>
+TCCL_D T* peer_words(const CommArgs& a, T* own, int rank) {
+  if (a.word_stride) return (T*)((char*)own + (int64_t)(rank - a.rank) * a.word_stride);
+  return translate_ptr(own, a.rank, rank, a.heap_bases);
+}
 
 // A rectangle to move.  Offsets are relative to a slice base.
 struct Xfer {
@@ -389,7 +400,7 @@ struct Waiter {
   TCCL_D bool tile(int tile_id, int rank) const {
     bool ok = true;
     if (threadIdx.x == 0) {
-      const int32_t* w = translate_ptr(a.locks, a.rank, rank, a.heap_bases);
+      const int32_t* w = peer_words(a, a.locks, rank);
       ok = tile_wait_ge<true>(w, tile_id, a.epoch, deadline);
     }
     return finish(ok);
@@ -401,7 +412,7 @@ struct Waiter {
     if (threadIdx.x == 0) {
       const int32_t need = a.epoch * a.tile_counts[g];
       for (int r = 0; r < a.world && ok; ++r)
-        if ((ranks >> r) & 1u) ok = tile_wait_ge<true>(translate_ptr(a.counter, a.rank, r, a.heap_bases), g, need, deadline);
+        if ((ranks >> r) & 1u) ok = tile_wait_ge<true>(peer_words(a, a.counter, r), g, need, deadline);
       if (ok && a.trace_ready_clock) {
         unsigned long long* slot = (unsigned long long*)&a.trace_ready_clock[g];
         atomicCAS(slot, 0ull, (unsigned long long)now_ticks());

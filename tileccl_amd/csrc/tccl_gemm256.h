@@ -146,6 +146,7 @@ struct PullArgs {
   int64_t* trace_done_clock;
   int64_t* fault;
   int64_t spin_ticks;
+  int64_t word_stride;         // as in CommArgs: 0 = a peer's counters sit in its heap slice
 };
 constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter word per wavefront (64 lanes x 4 B)
 
@@ -523,7 +524,8 @@ struct Gemm256 {
     const int64_t rel = ((int64_t)(uintptr_t)a->src0 - mine) + (int64_t)peer * a->block_bytes;
     st.src_base = theirs + rel;
     st.dst_base = mine + rel;
-    st.counter_base = (int64_t)(uintptr_t)a->counter + (theirs - mine);
+    const int64_t stride = a->word_stride;
+    st.counter_base = (int64_t)(uintptr_t)a->counter + (stride ? (int64_t)(peer - a->rank) * stride : theirs - mine);
     st.row0 = 0;  // the plan numbers the rows of one block
     st.gidx = 0;
     pull_group_facts(st, a);
