@@ -107,6 +107,12 @@ TCCL_D void st16(__amdgpu_buffer_rsrc_t w, uint32_t off, u32x4 v) { __builtin_am
 
 constexpr int kThreadsComm = 256;  // threads of a stand-alone communication workgroup
 constexpr int kCommUnroll = 8;     // 16-byte accesses a thread keeps in flight
+// Cache policy of the stand-alone bulk kernels (the second kernel of S0), measured on the
+// 128 MiB exchange that follows the 4096 x 4096 x 1024 GEMM and on the reductions of the
+// reduce-scatter configurations: plain (write-back) accesses for copies, 25.5 us against
+// 29.8 us with nt; nt for reductions (8192 x 4096 fp32 partials: 66.4 us against 69.8 plain).
+constexpr int kBulkCopyPolicy = 0;
+constexpr int kBulkReducePolicy = kStreaming;
 
 // ---- copy: units [u_lo, u_hi) of the rectangle, one source slice, any number of targets ----
 // kPolicy is the cache policy of both sides: kCoherent inside fused launches (the source
@@ -219,9 +225,11 @@ TCCL_D void store8(__amdgpu_buffer_rsrc_t w, uint32_t off, const float (&f)[8]) 
 template <typename PT, typename OT, int kPolicy, int kThreads>
 TCCL_D void run_reduce_t(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   constexpr uint32_t kSrcUnit = 8 * sizeof(PT);
-  // Units a thread keeps in flight.  A 512-thread workgroup has its CU to itself (the tail of
-  // the large-tile kernel), so it must carry the loads that several small workgroups would.
-  constexpr int kReduceUnroll = kThreads >= 512 ? 4 : 2;
+  // Units a thread keeps in flight.  Measured on the bulk reductions of 8192 x 4096 fp32 and
+  // 16384 x 4096 bf16 partials with 4 workgroups of 256 threads per CU: 2 units 68.0 / 126.0 us,
+  // 4 units 66.4 / 114.3 us, 8 units 84.4 / 140.8 us (the registers of the widest path set the
+  // occupancy of the whole kernel).
+  constexpr int kReduceUnroll = 4;
   const int tid = threadIdx.x;
   const int dst_rank = __builtin_ctz(x.dst_ranks);
   const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[dst_rank] + x.dst_off);
@@ -267,7 +275,7 @@ TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
     case kBF16 * 4 + kF16: run_reduce_t<__bf16, _Float16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
     case kF16 * 4 + kBF16: run_reduce_t<_Float16, __bf16, kPolicy, kThreads>(a, x, u_lo, u_hi); break;
     case kF32 * 4 + kF32:  // the stand-alone reduction only: the fused launches write 16-bit shards
-      if constexpr (kPolicy == kStreaming) run_reduce_t<float, float, kPolicy, kThreads>(a, x, u_lo, u_hi);
+      if constexpr (kPolicy != kCoherent) run_reduce_t<float, float, kPolicy, kThreads>(a, x, u_lo, u_hi);
       break;
     default: break;
   }
@@ -280,12 +288,12 @@ TCCL_D void run_xfer(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
     if (fused)
       run_reduce<kCoherent, kThreads>(a, x, u_lo, u_hi);
     else
-      run_reduce<kStreaming, kThreads>(a, x, u_lo, u_hi);
+      run_reduce<kBulkReducePolicy, kThreads>(a, x, u_lo, u_hi);
   } else {
     if (fused)
       run_copy<kCoherent, kThreads>(a, x, u_lo, u_hi);
     else
-      run_copy<kStreaming, kThreads>(a, x, u_lo, u_hi);
+      run_copy<kBulkCopyPolicy, kThreads>(a, x, u_lo, u_hi);
   }
 }
 

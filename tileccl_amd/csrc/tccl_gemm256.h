@@ -113,11 +113,12 @@ struct ReduceArgs {
 
 // Background transfer: the pull half of an all-gather, carried out in the shadow of the K
 // loop (TileGroup variant): out[block of peer] <- the peer's copy of that block.
-// A peer's block is cut into pieces of 64 units of 16 bytes; wavefront w of the launch owns
-// pieces w, w + W, w + 2W, ... (W = wavefronts in the grid), so at any moment the grid sweeps a
-// contiguous stretch.  In every K step, behind the step's operand loads, a wavefront requests
-// its next piece into four registers; the step's barrier waits for this wave's loads anyway,
-// and mid-way through the following step the piece is stored.  A
+// A peer's block is cut into pieces of kPieceUnits units of 16 bytes; pulling wavefront w of
+// the launch (the kPullWaves older wavefronts of every workgroup, see below) owns pieces w,
+// w + W, w + 2W, ... (W = pulling wavefronts in the grid), so at any moment the grid sweeps a
+// contiguous stretch.  In every K step, behind the step's operand loads, such a wavefront
+// requests its next piece into registers; the step's barrier waits for this wave's loads
+// anyway, and mid-way through the following step the piece is stored.  A
 // piece is fetched only once
 // the TileGroups covering its rows are complete on the peer (counter[g] >= epoch *
 // tile_counts[g], the readiness rule of tileccl_v2/signal.py:43-66); that is found out by
@@ -136,7 +137,7 @@ struct PullArgs {
   uint32_t pitch;              // bytes per row
   uint32_t upr;                // 16-byte units per row
   uint32_t units;              // units per block (rows * upr)
-  int pieces;                  // pieces per block: ceil(units / 64)
+  int pieces;                  // pieces per block: ceil(units / kPieceUnits)
   // synchronisation
   const int32_t* counter;      // this rank's TileGroup counters; a peer's sit at the same slice offset
   const int32_t* row_ends;
@@ -149,6 +150,15 @@ struct PullArgs {
   int64_t word_stride;         // as in CommArgs: 0 = a peer's counters sit in its heap slice
 };
 constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter word per wavefront (64 lanes x 4 B)
+// Of a SIMD's two wavefronts the older one (wavefronts 0..3 of the workgroup) wins the matrix
+// pipe and reaches each K step's barrier early, while the younger one runs alone for the rest of
+// the step; scalar work of the younger one therefore delays the step, that of the older one is
+// covered by the younger one's MFMAs.  The background pull is carried by the older wavefronts
+// alone, two 16-byte units per lane and step, so that its bookkeeping runs once per 2 KiB and
+// only where it is covered.
+constexpr int kPullWaves = 4;                           // wavefronts of a workgroup that pull
+constexpr int kPullLoads = 2;                           // 16-byte units per lane and piece
+constexpr int kPieceUnits = 64 * kPullLoads;            // units per piece
 
 TCCL_HD TileCoord macro_coords(int id, const Macro& m) {
   const int per_band = m.rows_per_band * m.cols;
@@ -385,7 +395,7 @@ struct Gemm256 {
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
     int pend_mask;           // bit per slot (K step parity): a piece was requested into it and is not yet stored
-    u32x4 piece[2];          // the pieces themselves (slots are always named statically)
+    u32x4 piece[2][kPullLoads];  // the pieces themselves (slots are always named statically)
     int probe_off;           // this wavefront's counter landing words
     // The counter word, read out of the landing words right behind a K step's barrier: read
     // there, it is older than every operand fetch that follows, so using it never waits for those.
@@ -398,9 +408,9 @@ struct Gemm256 {
     uint32_t upr, pitch, units;
     int pieces, slots, n_groups;
     uint32_t adv_row, adv_col;   // what `stride` pieces add to (row, col)
-    uint32_t row, col;           // per lane: row / unit of this lane's unit of piece next_lp
-    uint32_t pend_off[2];        // per lane: byte offset of the pending piece inside its block; kNoUnit: the
-                                 // unit does not exist (the last piece of a block may be short)
+    uint32_t row[kPullLoads], col[kPullLoads];  // per lane: row / unit-in-row of this lane's units of piece next_lp
+    uint32_t pend_off[2][kPullLoads];  // per lane: byte offsets of the pending piece's units inside the block;
+                                       // kNoUnit: the unit does not exist (a block's last piece may be short)
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -417,9 +427,9 @@ struct Gemm256 {
     PullState st;
     const int w = uniform(wave);
     st.probe_off = w * 256;
-    st.stride = num_wgs * (kThreads256 / 64);
+    st.stride = num_wgs * kPullWaves;
     st.next_slot = 0;
-    st.next_lp = wg * (kThreads256 / 64) + w;
+    st.next_lp = wg * kPullWaves + w;
     st.slot = -1;
     st.gidx = 0;
     st.row0 = 0;
@@ -431,13 +441,17 @@ struct Gemm256 {
     st.backoff = 0;
     st.pend_mask = 0;
     st.probe_val = 0;
-    st.piece[0] = st.piece[1] = u32x4{0, 0, 0, 0};
-    st.active = pull_offset >= 0 && a->mode != kBgNone;
+#pragma unroll
+    for (int j = 0; j < kPullLoads; ++j) {
+      st.piece[0][j] = st.piece[1][j] = u32x4{0, 0, 0, 0};
+      st.row[j] = st.col[j] = 0;
+      st.pend_off[0][j] = st.pend_off[1][j] = 0;
+    }
+    st.active = pull_offset >= 0 && a->mode != kBgNone && w < kPullWaves;
     st.primed = false;
     st.upr = st.pitch = st.units = 0;
     st.pieces = st.slots = st.n_groups = 0;
-    st.adv_row = st.adv_col = st.row = st.col = 0;
-    st.pend_off[0] = st.pend_off[1] = 0;
+    st.adv_row = st.adv_col = 0;
     if (st.active) {
       st.upr = a->upr;
       st.pitch = a->pitch;
@@ -445,7 +459,7 @@ struct Gemm256 {
       st.pieces = a->pieces;
       st.slots = a->slots;
       st.n_groups = a->n_groups;
-      const uint32_t adv = (uint32_t)st.stride * 64u;
+      const uint32_t adv = (uint32_t)st.stride * (uint32_t)kPieceUnits;
       st.adv_row = adv / st.upr;
       st.adv_col = adv - st.adv_row * st.upr;
       pull_normalise(st, a);
@@ -456,17 +470,23 @@ struct Gemm256 {
 
   // (row, col) of this lane's unit of piece next_lp, by division: at the start and when a block is finished.
   TCCL_D void pull_locate(PullState& st) const {
-    const uint32_t u = (uint32_t)st.next_lp * 64u + (uint32_t)lane;
-    st.row = u / st.upr;
-    st.col = u - st.row * st.upr;
+#pragma unroll
+    for (int j = 0; j < kPullLoads; ++j) {
+      const uint32_t u = (uint32_t)st.next_lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane);
+      st.row[j] = u / st.upr;
+      st.col[j] = u - st.row[j] * st.upr;
+    }
   }
   // The same after next_lp += stride.
   TCCL_D void pull_advance(PullState& st) const {
-    st.row += st.adv_row;
-    st.col += st.adv_col;
-    if (st.col >= st.upr) {
-      st.col -= st.upr;
-      ++st.row;
+#pragma unroll
+    for (int j = 0; j < kPullLoads; ++j) {
+      st.row[j] += st.adv_row;
+      st.col[j] += st.adv_col;
+      if (st.col[j] >= st.upr) {
+        st.col[j] -= st.upr;
+        ++st.row[j];
+      }
     }
   }
 
@@ -498,9 +518,9 @@ struct Gemm256 {
     }
   }
 
-  // Row and 16-byte unit inside the row of this lane's unit of piece lp (row 0, unit 0 for idle lanes).
-  TCCL_D void pull_unit(PullPtr a, int lp, bool& valid, uint32_t& row, uint32_t& col) const {
-    const uint32_t u = (uint32_t)lp * 64u + (uint32_t)lane;
+  // Row and 16-byte unit inside the row of this lane's unit j of piece lp (row 0, unit 0 for idle lanes).
+  TCCL_D void pull_unit(PullPtr a, int lp, int j, bool& valid, uint32_t& row, uint32_t& col) const {
+    const uint32_t u = (uint32_t)lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane);
     valid = u < a->units;
     const uint32_t uu = valid ? u : 0u;  // idle lanes touch the block's first unit and store nothing
     row = uu / a->upr;
@@ -508,7 +528,7 @@ struct Gemm256 {
   }
 
   TCCL_D uint32_t pull_last_unit(PullPtr a, int lp) const {
-    const uint32_t last = (uint32_t)lp * 64u + 63u;
+    const uint32_t last = (uint32_t)lp * (uint32_t)kPieceUnits + (uint32_t)(kPieceUnits - 1);
     return last < a->units ? last : a->units - 1u;
   }
 
@@ -561,8 +581,12 @@ struct Gemm256 {
   TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return false;
     if (!(st.pend_mask & (1 << slot))) return false;
-    const uint32_t off = st.pend_off[slot];
-    if (off != kNoUnit) st16<kStreaming>(window(st.dst_base), off, st.piece[slot]);
+    const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
+#pragma unroll
+    for (int j = 0; j < kPullLoads; ++j) {
+      const uint32_t off = st.pend_off[slot][j];
+      if (off != kNoUnit) st16<kStreaming>(dst, off, st.piece[slot][j]);
+    }
     st.pend_mask &= ~(1 << slot);
     return true;
   }
@@ -611,12 +635,17 @@ struct Gemm256 {
       return false;
     }
     pull_probe(st, a, landing);  // look ahead: the next group's counters (issued before the piece, which stays the youngest load)
-    const uint32_t last = (uint32_t)st.next_lp * 64u + 63u;
+    const uint32_t first = (uint32_t)st.next_lp * (uint32_t)kPieceUnits;
+    const uint32_t last = first + (uint32_t)(kPieceUnits - 1);
     if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
-      const bool valid = (uint32_t)st.next_lp * 64u + (uint32_t)lane < st.units;
-      const uint32_t off = valid ? st.row * st.pitch + st.col * 16u : 0u;  // idle lanes touch the block's first unit
-      st.piece[slot] = ld16<kCoherent>(window(st.src_base), off);
-      st.pend_off[slot] = valid ? off : kNoUnit;
+      const __amdgpu_buffer_rsrc_t src = window(st.src_base);
+#pragma unroll
+      for (int j = 0; j < kPullLoads; ++j) {
+        const bool valid = first + (uint32_t)(64 * j + lane) < st.units;
+        const uint32_t off = valid ? st.row[j] * st.pitch + st.col[j] * 16u : 0u;  // idle lanes touch the block's first unit
+        st.piece[slot][j] = ld16<kCoherent>(src, off);
+        st.pend_off[slot][j] = valid ? off : kNoUnit;
+      }
       st.pend_mask |= 1 << slot;
       st.next_lp += st.stride;
       if (st.next_lp >= st.pieces) {  // block finished: rare, may divide
@@ -650,47 +679,9 @@ struct Gemm256 {
   // After the last tile: finish what is in flight, move the remaining pieces, report.
   TCCL_D void pull_finish(PullState& st, PullPtr a, const char* landing, int num_wgs) const {
     if constexpr (kWithReduce) return;
-    if (!st.active) return;
-    wait_vmem();
-    pull_retire(st, a, landing, 0);
-    pull_retire(st, a, landing, 1);
-    st.probe_group = -1;
-    const int64_t deadline = now_ticks() + a->spin_ticks;
+    if (pull_offset < 0 || a->mode == kBgNone) return;  // the same for every wavefront: a barrier follows
     bool ok = true;
-    constexpr int kBatch = 8;  // pieces in flight per wavefront: the CU has no other work left
-    while (ok && st.next_slot < a->slots) {
-      pull_select(st, a, st.next_slot);
-      u32x4 v[kBatch];
-      uint32_t row[kBatch], col[kBatch];
-      bool valid[kBatch], loaded[kBatch];
-      int n = 0;
-#pragma unroll
-      for (int k = 0; k < kBatch; ++k) {
-        valid[k] = loaded[k] = false;
-        const int lp = st.next_lp + k * st.stride;
-        if (ok && lp < a->pieces) {
-          ok = pull_wait_ready(st, a, pull_last_unit(a, lp), deadline);
-          if (ok) {
-            pull_unit(a, lp, valid[k], row[k], col[k]);
-            const uint32_t off = row[k] * a->pitch + col[k] * 16u;
-            v[k] = ld16<kCoherent>(window(st.src_base), off);
-            loaded[k] = true;
-            n = k + 1;
-          }
-        }
-      }
-#pragma unroll
-      for (int k = 0; k < kBatch; ++k) {
-        if (loaded[k] && valid[k]) st16<kStreaming>(window(st.dst_base), row[k] * a->pitch + col[k] * 16u, v[k]);
-      }
-      st.next_lp += n * st.stride;
-      if (n < kBatch) {  // the block is finished (or a wait gave up)
-        st.next_lp -= a->pieces;
-        if (st.next_lp < 0) st.next_lp = 0;  // only after a failed wait
-        ++st.next_slot;
-        pull_normalise(st, a);
-      }
-    }
+    if (st.active) ok = pull_drain(st, a, landing);
     if (!ok && lane == 0 && a->fault) *a->fault = 1;
     wait_vmem();
     __syncthreads();
@@ -708,6 +699,62 @@ struct Gemm256 {
         }
       }
     }
+  }
+
+  // The pulling wavefronts' part of pull_finish; false if a bounded wait expired.
+  TCCL_D bool pull_drain(PullState& st, PullPtr a, const char* landing) const {
+    wait_vmem();
+    pull_retire(st, a, landing, 0);
+    pull_retire(st, a, landing, 1);
+    st.probe_group = -1;
+    const int64_t deadline = now_ticks() + a->spin_ticks;
+    bool ok = true;
+    constexpr int kBatch = 8;  // pieces in flight per pulling wavefront: the CU has no other work left
+    while (ok && st.next_slot < a->slots) {
+      pull_select(st, a, st.next_slot);
+      u32x4 v[kBatch][kPullLoads];
+      uint32_t off[kBatch][kPullLoads];
+      bool loaded[kBatch];
+      int n = 0;
+      const __amdgpu_buffer_rsrc_t src = window(st.src_base);
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        loaded[k] = false;
+        const int lp = st.next_lp + k * st.stride;
+        if (ok && lp < a->pieces) {
+          ok = pull_wait_ready(st, a, pull_last_unit(a, lp), deadline);
+          if (ok) {
+#pragma unroll
+            for (int j = 0; j < kPullLoads; ++j) {
+              bool valid;
+              uint32_t row, col;
+              pull_unit(a, lp, j, valid, row, col);
+              const uint32_t o = row * a->pitch + col * 16u;
+              v[k][j] = ld16<kCoherent>(src, o);
+              off[k][j] = valid ? o : kNoUnit;
+            }
+            loaded[k] = true;
+            n = k + 1;
+          }
+        }
+      }
+      const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        if (!loaded[k]) continue;
+#pragma unroll
+        for (int j = 0; j < kPullLoads; ++j)
+          if (off[k][j] != kNoUnit) st16<kStreaming>(dst, off[k][j], v[k][j]);
+      }
+      st.next_lp += n * st.stride;
+      if (n < kBatch) {  // the block is finished (or a wait gave up)
+        st.next_lp -= a->pieces;
+        if (st.next_lp < 0) st.next_lp = 0;  // only after a failed wait
+        ++st.next_slot;
+        pull_normalise(st, a);
+      }
+    }
+    return ok;
   }
 
   // 16-bit operand registers; they live across K steps.
