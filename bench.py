@@ -128,7 +128,7 @@ def launch_spread(run, variant, launches=100):
 class Workload:
     """One benchmark configuration: heap slices, resident inputs, the fused operation."""
 
-    def __init__(self, name, macro_tile):
+    def __init__(self, name, macro_tile, group_tiles=None):
         import torch
 
         from tileccl_amd.v2 import FusedGemmAllGather, FusedGemmReduceScatter, SymmetricHeap
@@ -136,6 +136,7 @@ class Workload:
         self.name = name
         self.kind, self.M, self.N, self.K, self.block_m, self.in_type = WORKLOADS[name]
         M, N, K = self.M, self.N, self.K
+        self.group_tiles, self.calibration = self.resolve_group_tiles(group_tiles)
         self.scales = (1.0, 1.0)
         if self.in_type == "f8":
             self.A_cpu, sa = quantised((M, K), 0, 1.0)
@@ -144,7 +145,7 @@ class Workload:
         else:
             self.A_cpu, self.B_cpu = seeded((M, K), 0), seeded((K, N), 1, K**-0.5)
         self.heaps = SymmetricHeap.create_all(2 << 30, 2)
-        common = dict(block_m=self.block_m, macro_tile=macro_tile)
+        common = dict(block_m=self.block_m, macro_tile=macro_tile, target_group_tiles=self.group_tiles)
         if self.kind == "ag":
             self.peer_cpu = seeded((M, N), 2)
             self.ops = [FusedGemmAllGather(h, M, N, torch.float16, directions="both", **common) for h in self.heaps]
@@ -179,6 +180,30 @@ class Workload:
         self.op.mark_peers_ready()
         self.flop = 2.0 * M * N * K
         self.own_out = {}
+
+    def resolve_group_tiles(self, group_tiles):
+        """`--group-tiles`: None keeps the planner's own rule (groups of at least tau_min bytes),
+        an integer is passed through, "auto" measures this machine and asks the cost model
+        (calibrate -> choose_target_group_tiles, the reference's "Phase0 calibration")."""
+        if group_tiles in (None, "default"):
+            return None, None
+        if group_tiles != "auto":
+            return int(group_tiles), None
+        from tileccl_amd.v2 import SymmetricHeap
+        from tileccl_amd.v2.calibrate import calibrate
+
+        heaps = SymmetricHeap.create_all(256 << 20, 2)  # its own slices: the workload's offsets stay symmetric
+        try:
+            cal = calibrate(heaps[0], gemm_shape=(self.M, self.N, self.K))
+        finally:
+            for h in heaps:
+                h.cleanup()
+        # the element type of what travels: the fp16 output block, or the partial of a reduce-scatter
+        dtype = "float16" if self.kind == "ag" else ("bfloat16" if self.in_type == "f8" else "float32")
+        tiles = cal.target_group_tiles(self.M, self.N, self.K, block_m=self.block_m, dtype=dtype)
+        return tiles, {"alpha_us": round(cal.profile.alpha_us, 3), "gbytes_per_s": round(1e-3 / cal.profile.beta_us_per_byte, 1),
+                       "launch_floor_us": round(cal.profile.min_comm_us, 3), "gemm_tflops": round(cal.gemm_tflops, 1),
+                       "in_launch_alpha_us": round(cal.in_launch_profile().alpha_us, 3), "target_group_tiles": tiles}
 
     def run(self, variant):
         self.op(self.A, self.B, variant, scale_a=self.scales[0], scale_b=self.scales[1])
@@ -379,6 +404,9 @@ def main() -> int:
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--macro-tile", type=int, default=0, choices=[0, 128, 256],
                     help="GEMM tile: 0 lets the library choose, 128 / 256 force a kernel")
+    ap.add_argument("--group-tiles", default="default",
+                    help="tiles per TileGroup: 'default' (the planner's rule), 'auto' (calibrate this machine and ask the "
+                         "cost model), or a number")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -391,7 +419,10 @@ def main() -> int:
 
     _lib.load()
     props = get_backend().get_device_properties()
-    w = (ChainedWorkload if WORKLOADS[args.workload][0] == "ch" else Workload)(args.workload, args.macro_tile)
+    if WORKLOADS[args.workload][0] == "ch":
+        w = ChainedWorkload(args.workload, args.macro_tile)
+    else:
+        w = Workload(args.workload, args.macro_tile, args.group_tiles)
 
     results = {}
     wanted = [v for v in ("s0", "s1", "s2") if v in args.variants.split(",") or v == args.variant]
@@ -434,6 +465,7 @@ def main() -> int:
         "config": {
             "workload": w.describe(args.variant),
             "tile_groups": w.op.plan.n_groups,
+            "group_tiles": w.op.plan.tile_counts()[0],
             "device": props.name,
             "compute_units": props.compute_units,
         },
@@ -449,10 +481,13 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.variant, args.macro_tile)),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.variant, args.macro_tile))
+            if args.group_tiles == "default" else None,
             "kernel_ms": round(chosen["event_ms_mean"], 5),
         },
     }
+    if getattr(w, "calibration", None):
+        line["config"]["calibration"] = w.calibration
     if push_only is not None:
         line["one_direction"] = push_only
     if "s0" in results and "s2" in results:

@@ -121,3 +121,26 @@ def test_choose_target_group_tiles_feeds_the_planner():
     slow = TileCostModel(HardwareProfile(alpha_us=500.0, beta_us_per_byte=1e-6, gemm_tflops_fp16=2500.0))
     fast = TileCostModel(HardwareProfile(alpha_us=0.1, beta_us_per_byte=1e-7, gemm_tflops_fp16=2500.0))
     assert choose_target_group_tiles(slow, 16384, 4096, 1024) >= choose_target_group_tiles(fast, 16384, 4096, 1024)
+
+
+def test_group_size_rule_prices_a_group_inside_a_launch_without_the_launch():
+    """Calibration points are stand-alone launches: ~7 us of latency that a TileGroup moved by a
+    running kernel does not pay.  Priced with it, one huge group wins (fewest launches); priced
+    without it, groups stay as small as the saturation floor allows, so that they pipeline."""
+    from tileccl_amd.v2.calibrate import Calibration
+    from tileccl_amd.v2.cost_model import HardwareProfile
+
+    prof = HardwareProfile(alpha_us=7.6, beta_us_per_byte=1e6 / 7.0e12, gemm_tflops_fp16=2500.0, gemm_efficiency=0.4,
+                           min_comm_us=7.2, name="measured")
+    cal = Calibration((), prof, 1000.0, int(7.6 / prof.beta_us_per_byte))
+    inside = cal.in_launch_profile()
+    assert inside.alpha_us == pytest.approx(0.4) and inside.min_comm_us == 0.0
+    assert inside.beta_us_per_byte == prof.beta_us_per_byte
+    # 8192 x 4096, 128 x 128 tiles: 8 swizzle waves of 256 tiles
+    assert cal.target_group_tiles(8192, 4096, 1024, in_launch=False) == 2048
+    assert cal.target_group_tiles(8192, 4096, 1024) == 256
+    assert cal.target_group_tiles(8192, 4096, 1024, block_m=256) == 256
+    # a link with real latency (xGMI-like: 2 us, 150 GB/s) asks for larger groups
+    slow = HardwareProfile(alpha_us=9.2, beta_us_per_byte=1e6 / 150e9, gemm_tflops_fp16=2500.0, gemm_efficiency=0.4,
+                           min_comm_us=7.2, name="link")
+    assert Calibration((), slow, 1000.0, 1).target_group_tiles(8192, 4096, 1024) >= 256

@@ -243,3 +243,52 @@ def test_argument_errors(lib):
     finally:
         for h in heaps:
             h.cleanup()
+
+
+@pytest.mark.parametrize("block_m", [128, 256])
+def test_baseline_config_2_with_the_group_size_chosen_by_the_cost_model(lib, block_m):
+    """Config 2 as it is worded: the TileGroup size comes from the cost model, fitted to
+    transfers and a GEMM measured on this machine (calibrate -> choose_target_group_tiles ->
+    build_tile_group_plan).  Whatever size comes out, S2 must move the bytes of the bulk
+    variant, match the oracle on a slab and leave every group's counter at its tile count."""
+    from tileccl_amd.v2 import SymmetricHeap
+    from tileccl_amd.v2.calibrate import calibrate
+
+    M, N, K = 8192, 4096, 1024
+    cal_heaps = SymmetricHeap.create_all(256 << 20, 2)
+    try:
+        cal = calibrate(cal_heaps[0], gemm_shape=(M, N, K))
+    finally:
+        for h in cal_heaps:
+            h.cleanup()
+    chosen = cal.target_group_tiles(M, N, K, block_m=block_m)
+    wave = 8 * (N // 128)
+    assert chosen % wave == 0 and wave <= chosen <= (M // block_m) * (N // 128)  # whole swizzle waves
+    assert cal.tau_min_bytes > 0 and cal.profile.beta_us_per_byte > 0
+    heaps, ops = make(2, M, N, heap_bytes=1 << 30, block_m=block_m, target_group_tiles=chosen)
+    try:
+        op = ops[0]
+        assert op.plan.target_group_tiles == chosen
+        assert all(n >= chosen for n in op.plan.tile_counts()[:-1]) and sum(op.plan.tile_counts()) == (M // block_m) * (N // 128)
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
+        peer = seeded((M, N), 2)
+        results = {}
+        for variant in ("s0", "s2"):
+            op.out.zero_()
+            ops[1].out.zero_()
+            ops[1].out[M:].copy_(peer)
+            op.mark_peers_ready()
+            op(A, B, variant)
+            op.check_faults()
+            assert torch.equal(bits(op.out), bits(op.peer_out(1))), variant
+            assert torch.equal(bits(op.out[M:]).cpu(), bits(peer)), variant
+            results[variant] = op.out[:M].clone()
+        assert torch.equal(bits(results["s0"]), bits(results["s2"]))
+        rows = slice(4000, 4128)
+        want = oracle.gemm(A_cpu[rows], B_cpu, torch.float16)
+        assert (results["s2"][rows].float().cpu() - want.float()).abs().max().item() <= 0.004
+        assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
+    finally:
+        for h in heaps:
+            h.cleanup()

@@ -94,9 +94,28 @@ class Calibration:
     def model(self) -> TileCostModel:
         return TileCostModel(self.profile)
 
-    def target_group_tiles(self, M: int, N: int, K: int, **kwargs) -> int:
-        kwargs.setdefault("tau_min_bytes", self.tau_min_bytes)
-        return choose_target_group_tiles(self.model(), M, N, K, **kwargs)
+    def in_launch_profile(self) -> HardwareProfile:
+        """The fitted link as a transfer inside a fused launch sees it.
+
+        The measured points are stand-alone launches, so their latency term is dominated by
+        the launch itself (the fit's floor, ~7 us here); a TileGroup moved by a launch that is
+        already running pays only what exceeds that floor.  Bandwidth is unchanged.
+        """
+        p = self.profile
+        alpha = max(p.alpha_us - p.min_comm_us, 0.05)
+        return HardwareProfile(alpha_us=alpha, beta_us_per_byte=p.beta_us_per_byte, gemm_tflops_fp16=p.gemm_tflops_fp16,
+                               gemm_efficiency=p.gemm_efficiency, min_comm_us=0.0, name=f"{p.name}, inside a launch")
+
+    def target_group_tiles(self, M: int, N: int, K: int, *, in_launch: bool = True, **kwargs) -> int:
+        """``target_group_tiles`` for ``build_tile_group_plan``; ``in_launch`` prices a group's
+        transfer without the launch latency (the fused S1 / S2 kernels), otherwise as a
+        stand-alone launch per group."""
+        if not in_launch:
+            kwargs.setdefault("tau_min_bytes", self.tau_min_bytes)
+            return choose_target_group_tiles(self.model(), M, N, K, **kwargs)
+        prof = self.in_launch_profile()
+        kwargs.setdefault("tau_min_bytes", max(int(prof.alpha_us / prof.beta_us_per_byte), 1))
+        return choose_target_group_tiles(TileCostModel(prof), M, N, K, **kwargs)
 
 
 def calibrate(heap: SymmetricHeap, *, gemm_shape: tuple[int, int, int] = (4096, 4096, 1024),
