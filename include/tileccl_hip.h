@@ -90,7 +90,11 @@ typedef struct tccl_gemm_desc {
   int32_t num_wgs;   /* GEMM workgroups; 0 = library default for the device */
   int32_t macro_tile; /* output tile one workgroup computes: 0 = choose by shape, 128, or 256 */
   int32_t flags;      /* TCCL_GEMM_* bits */
-  int32_t reserved;
+  /* Column shards stacked as row blocks (the rank_major_column_shards layout of
+   * tileccl.ops.gemm_reducescatter, ops.py:315,646).  0 or 1: plain GEMM.  w > 1: A has M/w
+   * rows and B has w*N columns; row block q of C (rows [q*M/w, (q+1)*M/w)) is
+   * A @ B[:, q*N:(q+1)*N].  M/w must be a multiple of the plan tile's rows. */
+  int32_t column_shards;
 } tccl_gemm_desc;
 
 /* tccl_gemm_reducescatter, variants S1 / S2 on the 256 x 256 tile with shards of whole tiles:
@@ -100,6 +104,9 @@ typedef struct tccl_gemm_desc {
  * (The reference's fused proof kernels have no counterpart in its tree; tile_reduce_scatter,
  * primitives/collectives.py:730-783, always reads a stored partial.) */
 #define TCCL_GEMM_OWN_ROWS_IN_REGISTERS 1
+
+#define TCCL_RS_EMULATE_PEERS 1
+#define TCCL_RS_PEERS_RESIDENT 2
 
 /* ---- per-launch synchronisation words ------------------------------------------------
  * Stands in for the lock tensor of WGSpecializedPattern (wg_specialized.py:104-124) and
@@ -278,7 +285,11 @@ int tccl_gemm_allgather(const tccl_gemm_desc* gemm, void* out, int64_t ld_out,
                         const tccl_transport_desc* transport, int32_t variant, void* stream);
 
 /* GEMM to ReduceScatter (Gate 2).  gemm->C is the rank's partial (M x N, dtype
- * gemm->out_dtype) in its slice; `out` receives the rank's M/world_size row shard. */
+ * gemm->out_dtype) in its slice; `out` receives the rank's M/world_size row shard.
+ * emulate_peer is a bit mask: TCCL_RS_EMULATE_PEERS also carries out the other owners'
+ * reductions into their slices (the whole operation on one GPU); TCCL_RS_PEERS_RESIDENT
+ * declares the peers' partials complete in memory, so that no launch waits for their signal
+ * words (ranks emulated one after another in one process, where a peer cannot be running). */
 int tccl_gemm_reducescatter(const tccl_gemm_desc* gemm, void* out, int32_t out_dtype, int64_t ld_out,
                             const tccl_heap_view* heap, const tccl_sync_desc* sync,
                             const tccl_transport_desc* transport, int32_t emulate_peer,

@@ -51,11 +51,18 @@ def test_gemm_allgather_column_shards(lib, variant, world, M, N, K):
             c.heap.cleanup()
 
 
-@pytest.mark.parametrize("world,M,N,K", [(2, 512, 512, 256), (2, 200, 272, 72), (3, 256, 768, 128)])
-def test_gemm_reducescatter_column_shards(lib, world, M, N, K):
+@pytest.mark.parametrize("variant", ["s0", "s1", "s2"])
+@pytest.mark.parametrize("world,M,N,K", [(2, 512, 512, 256), (2, 200, 272, 72), (3, 256, 768, 128), (2, 2048, 4096, 512),
+                                         (3, 768, 1536, 192)])
+def test_gemm_reducescatter_column_shards(lib, variant, world, M, N, K):
+    """One fused launch per rank (GEMM over the stacked column blocks + reduction of the own
+    block), M = 200 being the shape that falls back to one GEMM per block plus the bulk
+    reduction.  First with every partial stored, so that the oracle can reduce the very
+    partials the GPU produced (bit-exact for two ranks); then in the default mode, where the
+    own block's partial stays in the accumulators: same output bytes."""
     import tileccl_amd as tileccl
 
-    ctxs = contexts(world)
+    ctxs = contexts(world, 256 << 20)
     try:
         Ns = N // world
         A_cpu = [seeded((M, K), 10 + r) for r in range(world)]
@@ -67,12 +74,16 @@ def test_gemm_reducescatter_column_shards(lib, world, M, N, K):
         # after the second round every rank has reduced over final partials.
         for _ in range(2):
             for r, c in enumerate(ctxs):
-                assert tileccl.ops.gemm_reducescatter(As[r], Bs[r], Cs[r], ctx=c) is Cs[r]
+                out = tileccl.ops.gemm_reducescatter(As[r], Bs[r], Cs[r], ctx=c, variant=variant, own_rows_in_registers=False)
+                assert out is Cs[r]
         torch.cuda.synchronize()
         full = sum(a.float() @ B_cpu.float() for a in A_cpu)
         partials = [c.workspace("gemm_reducescatter.partial", world, M, Ns, dtype=torch.float32).cpu() for c in ctxs]
+        stored = [t.clone() for t in Cs]
         for r in range(world):
             assert_gemm_close(Cs[r], full[:, r * Ns:(r + 1) * Ns], tight=0.006)
+            for q in range(world):  # block q of rank r's workspace is A_r @ B[:, q's columns]
+                assert_gemm_close(partials[r][q], A_cpu[r].float() @ B_cpu[:, q * Ns:(q + 1) * Ns].float(), tight=1e-3)
             # bit-exact against the oracle's reduction of the partials the GPU produced
             tall = [p.reshape(world * M, Ns) for p in partials]
             want = oracle.reduce_rows(tall, r, torch.float16)
@@ -80,6 +91,24 @@ def test_gemm_reducescatter_column_shards(lib, world, M, N, K):
                 assert torch.equal(bits(Cs[r]).cpu(), bits(want))
             else:
                 assert (Cs[r].cpu().float() - want.float()).abs().max().item() <= 0.002
+        # Default mode: the own block's partial is never stored; the peers' blocks are.
+        for r, c in enumerate(ctxs):
+            c.workspace("gemm_reducescatter.partial", world, M, Ns, dtype=torch.float32)[r].fill_(-3.0)
+            Cs[r].zero_()
+        for r, c in enumerate(ctxs):
+            tileccl.ops.gemm_reducescatter(As[r], Bs[r], Cs[r], ctx=c, variant=variant)
+        torch.cuda.synchronize()
+        fused = M % 128 == 0 and variant != "s0"
+        for r, c in enumerate(ctxs):
+            assert torch.equal(bits(Cs[r]), bits(stored[r])), r
+            mine = c.workspace("gemm_reducescatter.partial", world, M, Ns, dtype=torch.float32)
+            # the large-tile kernel (chosen from 128 tiles of 256 x 256 on) is the one that keeps rows in registers
+            macro = M % 256 == 0 and -(-world * M // 256) * -(-Ns // 256) * 2 >= 256
+            if fused and macro:
+                assert torch.all(mine[r] == -3.0), r
+            for q in range(world):
+                if q != r:
+                    assert torch.equal(mine[q].cpu(), partials[r][q]), (r, q)
     finally:
         for c in ctxs:
             c.heap.cleanup()

@@ -65,6 +65,7 @@ def gemm_desc(
     num_wgs: int = 0,
     macro_tile: int = 0,
     flags: int = 0,
+    column_shards: int = 0,
 ) -> _lib.GemmDesc:
     if not (A.is_cuda and B.is_cuda and C_out.is_cuda):
         raise ValueError("GEMM operands must be device tensors")
@@ -74,6 +75,10 @@ def gemm_desc(
     K2, N = B.shape
     if K2 != K:
         raise ValueError(f"B.shape[0] must equal A.shape[1]: got {K2} vs {K}")
+    if column_shards > 1:  # C stacks the column blocks of A @ B as row blocks
+        if N % column_shards:
+            raise ValueError(f"B.shape[1]={N} must be divisible by column_shards={column_shards}")
+        M, N = M * column_shards, N // column_shards
     if tuple(C_out.shape) != (M, N):
         raise ValueError(f"C shape mismatch: expected ({M}, {N}), got {tuple(C_out.shape)}")
     d = _lib.GemmDesc()
@@ -86,6 +91,7 @@ def gemm_desc(
     d.num_wgs = int(num_wgs)
     d.macro_tile = int(macro_tile)
     d.flags = int(flags)
+    d.column_shards = int(column_shards)
     return d
 
 

@@ -22,6 +22,7 @@ S0_BULK, S1_TILE, S2_TILEGROUP = 0, 1, 2
 DIR_PUSH, DIR_PULL = 1, 2
 ERR_INVALID, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_TIMEOUT = -1, -2, -3, -4
 MAX_WORLD = 8
+RS_EMULATE_PEERS, RS_PEERS_RESIDENT = 1, 2
 
 
 class DeviceInfo(C.Structure):
@@ -56,7 +57,7 @@ class GemmDesc(C.Structure):
         ("num_wgs", C.c_int32),
         ("macro_tile", C.c_int32),
         ("flags", C.c_int32),
-        ("reserved", C.c_int32),
+        ("column_shards", C.c_int32),
     ]
 
 

@@ -184,16 +184,21 @@ int check_gemm(const tccl_gemm_desc* d) {
   if (d->in_dtype == TCCL_F8E4M3 && (d->macro_tile == 128 || !plan_tile_fits_macro(d)))
     return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 inputs need the 256x256 kernel (macro_tile 0 or 256, plan tile edges 128 or 256)");
   if (d->out_dtype == TCCL_F8E4M3) return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 output is not supported");
+  const int shards = d->column_shards > 1 ? d->column_shards : 1;
+  if (d->column_shards < 0 || d->M % shards || (shards > 1 && (d->M / shards) % d->block_m))
+    return fail(TCCL_ERR_INVALID, "gemm: column_shards=%d must split M=%d into blocks of whole %d-row plan tiles", d->column_shards, d->M, d->block_m);
+  if (d->in_dtype == TCCL_F8E4M3 && shards > 1 && (d->M / shards) % 256)
+    return fail(TCCL_ERR_UNSUPPORTED, "gemm: fp8 inputs with column_shards need row blocks of whole 256-row tiles");
   const int in_vec = (int)(16 / isz), out_vec = (int)(16 / osz);
   if (d->K % in_vec) return fail(TCCL_ERR_UNSUPPORTED, "gemm: K=%d must be a multiple of %d", d->K, in_vec);
   if (d->N % 8) return fail(TCCL_ERR_UNSUPPORTED, "gemm: N=%d must be a multiple of 8", d->N);
-  if (d->lda < d->K || d->ldb < d->N || d->ldc < d->N) return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
+  if (d->lda < d->K || d->ldb < (int64_t)d->N * shards || d->ldc < d->N) return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
   if (d->lda % in_vec || d->ldb % in_vec || d->ldc % out_vec || !aligned16(d->A) || !aligned16(d->B) || !aligned16(d->C))
     return fail(TCCL_ERR_UNSUPPORTED, "gemm: A, B, C rows must start on 16-byte boundaries");
   // The kernels address an operand with 32-bit byte offsets from a per-tile base: B from its
   // first row down to row K-1, A and C over the 256 rows of a tile.
   const int64_t limit = 0xffffffffll;
-  const int64_t b_span = ((int64_t)(d->K - 1) * d->ldb + d->N) * (int64_t)isz;
+  const int64_t b_span = ((int64_t)(d->K - 1) * d->ldb + (int64_t)d->N * shards) * (int64_t)isz;
   const int64_t a_span = (255 * d->lda + d->K) * (int64_t)isz;
   const int64_t c_span = (255 * d->ldc + d->N) * (int64_t)osz;
   if (b_span > limit || a_span > limit || c_span > limit)
@@ -230,6 +235,7 @@ int build_gemm_args(const tccl_gemm_desc* d, const tccl_device_info& dev, tccl::
   g->tile_cols = (d->N + d->block_n - 1) / d->block_n;
   g->xcds = dev.xcds;
   g->span = gemm_span(d->group_m * g->tile_cols, d->group_m, g->tile_cols, dev.xcds);
+  g->wrap_rows = d->column_shards > 1 ? d->M / d->column_shards : 0;
   return 0;
 }
 
@@ -334,6 +340,7 @@ int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tcc
 bool use_macro(const tccl_gemm_desc* d, const tccl_device_info& dev) {
   if (d->in_dtype == TCCL_F8E4M3) return true;  // fp8 exists only as the large-tile kernel (check_gemm vets the plan tile)
   if (!plan_tile_fits_macro(d)) return false;
+  if (d->column_shards > 1 && (d->M / d->column_shards) % 256) return false;  // a tile must not straddle two row blocks
   if (d->macro_tile == 128) return false;
   if (d->macro_tile == 256) return true;
   const int64_t tiles = (int64_t)((d->M + 255) / 256) * ((d->N + 255) / 256);
@@ -455,6 +462,7 @@ bool build_reduce(const tccl::CommArgs& c, const tccl_sync_desc* sync, int flags
   r->rank = c.rank;
   r->world = c.world;
   r->emulate_peer = c.emulate_peer;
+  r->peers_resident = c.peers_resident;
   r->shard_rows = shard;
   r->out_bf16 = c.out_dtype == tccl::kBF16;
   r->own_in_registers = (flags & TCCL_GEMM_OWN_ROWS_IN_REGISTERS) != 0;
@@ -988,7 +996,8 @@ static int fill_reduce(tccl::CommArgs* c, const void* partial, int partial_dtype
   c->ld_rs_out_bytes = ld_out * (out_dtype == TCCL_F32 ? 4 : 2);
   c->partial_dtype = partial_dtype;
   c->out_dtype = out_dtype;
-  c->emulate_peer = emulate_peer;
+  c->emulate_peer = (emulate_peer & TCCL_RS_EMULATE_PEERS) != 0;
+  c->peers_resident = (emulate_peer & TCCL_RS_PEERS_RESIDENT) != 0;
   // Without a plan the kernel works shard by shard (one implicit group per owner).
   if (!c->row_starts) c->n_groups = world;
   return 0;

@@ -57,6 +57,7 @@ struct CommArgs {
   char* rs_out;
   int64_t ld_rs_out_bytes;
   int partial_dtype, out_dtype, emulate_peer;
+  int peers_resident;  // reduce-scatter: the peers' partials are complete in memory, their words are not waited for
   // synchronisation words and TileGroups
   int32_t* locks;
   int32_t* counter;
@@ -406,6 +407,7 @@ struct Waiter {
   // S1: locks[tile] of `rank`'s slice has reached this launch's epoch (tile_publish).  The
   // word is only observed, whoever owns it: several parties may depend on the same tile.
   TCCL_D bool tile(int tile_id, int rank) const {
+    if (rank != a.rank && a.peers_resident) return true;
     bool ok = true;
     if (threadIdx.x == 0) {
       const int32_t* w = peer_words(a, a.locks, rank);
@@ -417,6 +419,7 @@ struct Waiter {
   // S2: counter[g] of every slice in `ranks` has reached epoch * tile_counts[g].
   TCCL_D bool group(int g, uint32_t ranks) const {
     bool ok = true;
+    if (a.peers_resident) ranks &= 1u << a.rank;
     if (threadIdx.x == 0) {
       const int32_t need = a.epoch * a.tile_counts[g];
       for (int r = 0; r < a.world && ok; ++r)

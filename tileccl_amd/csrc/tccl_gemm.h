@@ -54,7 +54,32 @@ struct GemmArgs {
   int block_m, block_n, group_m;  // plan tile and swizzle band
   int tile_rows, tile_cols;       // plan tiles
   int xcds, span;                 // slot -> tile remap
+  // Column shards stacked as row blocks (0: plain GEMM): C row block q of wrap_rows rows is
+  // A (wrap_rows x K) times columns [q * N, (q + 1) * N) of B; tiles never straddle two blocks.
+  int wrap_rows;
 };
+
+// Where a tile whose first output row is row0 and first output column col0 reads its operands.
+struct OperandOrigin {
+  int a_row, a_rows;  // first row of A, rows A has
+  int b_col, b_cols;  // first column of B, columns B has
+};
+TCCL_HD OperandOrigin operand_origin(const GemmArgs& g, int row0, int col0) {
+  OperandOrigin o;
+  if (g.wrap_rows > 0) {
+    const int q = row0 / g.wrap_rows;
+    o.a_row = row0 - q * g.wrap_rows;
+    o.a_rows = g.wrap_rows;
+    o.b_col = col0 + q * g.N;
+    o.b_cols = (g.M / g.wrap_rows) * g.N;
+  } else {
+    o.a_row = row0;
+    o.a_rows = g.M;
+    o.b_col = col0;
+    o.b_cols = g.N;
+  }
+  return o;
+}
 
 struct SignalArgs {
   int mode;
@@ -126,10 +151,11 @@ struct GemmRole {
   TCCL_D Source make_source(int row0, int col0) const {
     constexpr int kEsz = sizeof(InT);
     Source s;
-    const InT* A = (const InT*)g.A + (int64_t)row0 * g.lda;
-    const InT* B = (const InT*)g.B + col0;
-    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(g.M - 1 - row0) * g.lda + g.K) * kEsz), 0x00020000);
-    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (g.N - col0)) * kEsz), 0x00020000);
+    const OperandOrigin o = operand_origin(g, row0, col0);
+    const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
+    const InT* B = (const InT*)g.B + o.b_col;
+    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * kEsz), 0x00020000);
+    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       s.off_a[i] = (uint32_t)(((tid >> 3) + 32 * i) * g.lda * kEsz + (tid & 7) * 16);

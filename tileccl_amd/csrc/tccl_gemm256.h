@@ -97,6 +97,7 @@ struct PushArgs {
 struct ReduceArgs {
   int active;
   int rank, world, emulate_peer;
+  int peers_resident;             // the peers' partials are complete in memory: never wait for their words
   int shard_rows;                 // rows per owner; a multiple of the 256-row tile
   int out_bf16;                   // output element: 0 fp16, 1 bf16
   int own_in_registers;           // own rows: sum the peers' partials onto the accumulators, store no partial
@@ -264,10 +265,11 @@ struct Gemm256 {
   TCCL_D Source make_source(int row0, int col0) const {
     constexpr int kEsz = sizeof(InT);
     Source s;
-    const InT* A = (const InT*)g.A + (int64_t)row0 * g.lda;
-    const InT* B = (const InT*)g.B + col0;
-    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(g.M - 1 - row0) * g.lda + g.K) * kEsz), 0x00020000);
-    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (g.N - col0)) * kEsz), 0x00020000);
+    const OperandOrigin o = operand_origin(g, row0, col0);
+    const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
+    const InT* B = (const InT*)g.B + o.b_col;
+    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * kEsz), 0x00020000);
+    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = 8 * (4 * wave + i) + (lane >> 3);
@@ -1160,6 +1162,7 @@ struct Gemm256 {
   // Are the peers' partials of the plan tiles under macro tile (mm, mn) published?  One lane
   // waits (bounded); the verdict travels through an LDS word of the idle stage.
   TCCL_D bool reduce_wait(ReducePtr ra, const SignalArgs& s, int mm, int mn) const {
+    if (ra->peers_resident) return true;  // the same for every wavefront
     volatile int* verdict = (volatile int*)lds1;
     if (tid == 0) {
       bool ok = true;

@@ -172,18 +172,50 @@ def gemm_allgather(A: Any, B_shard: Any, Cx: Any, *, ctx=None, storage_kind: str
     return Cx
 
 
+def _reduce_scatter_words(ctx, world: int, M: int, cols: int):
+    """Signal words and TileGroup plan of the fused column-shard reduce-scatter, kept per shape
+    on the context.  Every rank allocates them in the same order, so a peer's words sit at the
+    same offset of its slice."""
+    from tileccl_amd.v2.tile_group import build_tile_group_plan
+
+    cache = ctx.__dict__.setdefault("_reduce_scatter_words", {})
+    key = (world, M, cols)
+    if key not in cache:
+        plan = build_tile_group_plan(world * M, cols, 128 * 128 * 4, row_split_boundaries=[M * q for q in range(1, world)])
+        heap = ctx.require_heap()
+        words = {name: heap.allocate_tensor((n,), torch.int32) for name, n in
+                 (("counter", plan.n_groups), ("barrier", plan.n_groups), ("locks", int(plan.group_table.numel())))}
+        for t in words.values():
+            t.zero_()
+        cache[key] = _launch.SyncWords(plan=_launch.DevicePlan.upload(plan), host_plan=plan, **words)
+    return cache[key]
+
+
 def gemm_reducescatter(A: Any, B: Any, Cx: Any, *, ctx=None, implementation: str = "auto",
-                       storage_kind: str = "symmetric", emulate_peer: bool = False) -> Any:
+                       storage_kind: str = "symmetric", emulate_peer: bool = False, variant: str = "s2",
+                       own_rows_in_registers: bool = True) -> Any:
     """``C = (sum over ranks of A_rank @ B)[:, this rank's columns]``.
 
     The partial products live in the context workspace ``"gemm_reducescatter.partial"`` of
     shape ``(world, M, N/world)``, fp32, at the same offset of every rank's slice; block
-    ``q`` is ``A @ B[:, q's columns]``.  ``emulate_peer`` (single-GPU emulation) also writes
-    the other ranks' outputs into their slices.  ``implementation`` is accepted for
-    signature parity; there is one implementation here.
+    ``q`` is ``A @ B[:, q's columns]`` (the reference's rank-major column-shard layout,
+    ops.py:315,646).  Stacked, the blocks are the row shards of a ``(world*M, N/world)``
+    matrix, so the operation is one launch of the fused GEMM -> ReduceScatter kernel: the
+    GEMM produces row block ``q`` from ``B``'s column block ``q``, block ``rank`` is reduced
+    with the peers' partials as its tiles finish, and (``own_rows_in_registers``, the default)
+    that block never leaves the accumulators as a partial, so its part of the workspace is not
+    written.  ``variant`` picks the schedule (``"s0"`` bulk, ``"s1"`` tile by tile, ``"s2"``
+    TileGroup).  ``emulate_peer`` (single-GPU emulation) also writes the other ranks' outputs
+    into their slices.  Ranks of this single-process build run one after another, so a launch
+    takes the peers' partials as resident and does not wait for their signals.
+    ``implementation`` is accepted for signature parity; there is one implementation here.
+    When ``M`` is not a multiple of the 128-row plan tile, one GEMM per column block and the
+    bulk reduction run instead.
     """
     if implementation not in ("auto", "device", "hip"):
         raise ValueError(f"unsupported gemm_reducescatter implementation {implementation!r}")
+    if variant not in _launch.VARIANTS:
+        raise ValueError(f"unknown variant {variant!r}; expected one of {sorted(_launch.VARIANTS)}")
     ctx = ctx if ctx is not None else tileccl_amd.current_context()
     k = resolve_gemm_reducescatter_contract(A, B, Cx, ctx=ctx, storage_kind=storage_kind)
     lib = _lib.load()
@@ -192,12 +224,27 @@ def gemm_reducescatter(A: Any, B: Any, Cx: Any, *, ctx=None, implementation: str
         _lib.check(lib.tccl_gemm(C.byref(_launch.gemm_desc(A, B, Cx)), stream), "tccl_gemm")
         return Cx
     partial = ctx.workspace("gemm_reducescatter.partial", k.world_size, k.M, k.output_cols, dtype=torch.float32)
-    for q in range(k.world_size):
-        cols = B[:, q * k.output_cols:(q + 1) * k.output_cols]
-        _lib.check(lib.tccl_gemm(C.byref(_launch.gemm_desc(A, cols, partial[q])), stream), "tccl_gemm")
     tall = partial.view(k.world_size * k.M, k.output_cols)  # row block q = the shard rank q owns
     view = _launch.heap_view(ctx.heap_bases, k.rank, k.world_size)
     transport = _launch.transport_desc(_lib.DIR_PULL, 16384, 16384, 0)
+    if k.M % 128 == 0:
+        words = _reduce_scatter_words(ctx, k.world_size, k.M, k.output_cols)
+        gemm = _launch.gemm_desc(A, B, tall, column_shards=k.world_size,
+                                 flags=_lib.GEMM_OWN_ROWS_IN_REGISTERS if own_rows_in_registers else 0)
+        if variant != "s0":
+            words.next_epoch(variant)
+        sync = words.desc(variant)
+        mode = _lib.RS_PEERS_RESIDENT | (_lib.RS_EMULATE_PEERS if emulate_peer else 0)
+        rc = lib.tccl_gemm_reducescatter(
+            C.byref(gemm), _launch.ptr(Cx), _launch.dtype_code(Cx.dtype), int(Cx.stride(0)), C.byref(view), C.byref(sync),
+            C.byref(transport), mode, _launch.VARIANTS[variant], stream,
+        )
+        _lib.check(rc, f"tccl_gemm_reducescatter[{variant}]")
+        ctx.__dict__["_reduce_scatter_last_words"] = words
+        return Cx
+    for q in range(k.world_size):
+        cols = B[:, q * k.output_cols:(q + 1) * k.output_cols]
+        _lib.check(lib.tccl_gemm(C.byref(_launch.gemm_desc(A, cols, partial[q])), stream), "tccl_gemm")
     rc = lib.tccl_reduce_rows(
         _launch.ptr(tall), _launch.dtype_code(tall.dtype), int(tall.stride(0)), _launch.ptr(Cx), _launch.dtype_code(Cx.dtype),
         int(Cx.stride(0)), int(tall.shape[0]), int(tall.shape[1]), C.byref(view), C.byref(transport), int(emulate_peer), stream,
