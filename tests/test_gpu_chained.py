@@ -32,7 +32,9 @@ def put(ctx, cpu):
     (1, 256, 64, 256, torch.float16),      # one rank: the gather is a plain copy, nothing is scattered
     (2, 512, 128, 512, torch.float16),
     (3, 300, 72, 264, torch.float16),      # ragged rows, K_shard not a multiple of the K step
-    (2, 4096, 512, 4096, torch.bfloat16),  # large-tile kernel
+    (2, 4096, 512, 4096, torch.bfloat16),  # large-tile kernel: the one-launch schedules read the shards in place
+    (3, 2048, 192, 4096, torch.float16),   # the same with three shards of three K steps each, odd step count
+    (2, 2048, 96, 4096, torch.float16),    # large-tile kernel, shards that are not whole K steps: gathered first
 ])
 def test_chained_matches_the_oracle(lib, schedule, world, M, Ks, N, dtype):
     from tileccl_amd.patterns.chained_ag_gemm_rs import ChainedAGGemmRSPattern

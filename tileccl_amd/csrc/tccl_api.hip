@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 
 #include "../../include/tileccl_hip.h"
 #include "tccl_comm.h"
@@ -122,10 +123,11 @@ struct Fused256Args {
   tccl::PullArgs pull;
   tccl::PushArgs push;
   tccl::ReduceArgs reduce;
+  tccl::GatherArgs gather;
   tccl::CommArgs comm;
 };
 
-template <typename InT, typename OutT, bool kWithReduce>
+template <typename InT, typename OutT, bool kWithReduce, bool kGatherA = false>
 __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
@@ -133,8 +135,9 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
   __shared__ __attribute__((aligned(16))) char landing_words[tccl::kBgWordBytes];
   tccl::warm_kernargs<(int)sizeof(Fused256Args)>();
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
-  tccl::Gemm256<InT, OutT, kWithReduce>(f.g, (int)offsetof(Fused256Args, pull), (int)offsetof(Fused256Args, push), (int)offsetof(Fused256Args, reduce), stage0, stage1,
-                                        landing_words)
+  tccl::Gemm256<InT, OutT, kWithReduce, kGatherA>(f.g, (int)offsetof(Fused256Args, pull), (int)offsetof(Fused256Args, push),
+                                                  (int)offsetof(Fused256Args, reduce), stage0, stage1, landing_words,
+                                                  (int)offsetof(Fused256Args, gather))
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();
   const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));
@@ -396,7 +399,13 @@ template <typename InT, typename OutT>
 int launch_fused256_t(const Fused256Args& f, int wgs, hipStream_t stream) {
   // The tile-by-tile reduce-scatter is a separate instantiation: its code would otherwise
   // raise the register pressure of every fused kernel.
-  if (f.reduce.active)
+  if (f.gather.active) {
+    // Instantiated for outputs of the input type only (gather_in_place() admits nothing else).
+    if constexpr (std::is_same<InT, OutT>::value)
+      hipLaunchKernelGGL((fused256_kernel<InT, OutT, false, true>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
+    else
+      return fail(TCCL_ERR_UNSUPPORTED, "gathered input read in place: output type must equal the input type");
+  } else if (f.reduce.active)
     hipLaunchKernelGGL((fused256_kernel<InT, OutT, true>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
   else
     hipLaunchKernelGGL((fused256_kernel<InT, OutT, false>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
@@ -533,9 +542,56 @@ int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
 // reductions of the reduce-scatter configurations (4 per CU ahead of 8 by 3-4 %).
 int bulk_comm_wgs(const tccl_device_info& dev) { return dev.compute_units * 4; }
 
+// The shards that make up the GEMM's A operand, when the chained operation reads them in place.
+struct GatherSpec {
+  const void* shard;
+  int64_t ld_shard;
+  int k_shard;
+};
+
+// Can the one-launch variants of the chained operation read the gathered input in place?
+// Large-tile kernel, 16-bit inputs and an output of the same type, shards of whole K steps.
+bool gather_in_place(const tccl_gemm_desc* d, const tccl_device_info& dev, int k_shard, int variant);
+
+// The background transfer that fills the gathered workspace (gemm->A) while the K loops run.
+void build_gather_background(const tccl_gemm_desc* d, const GatherSpec& gs, const tccl_heap_view* heap, const tccl::CommArgs& c,
+                             tccl::PullArgs* p, tccl::GatherArgs* ga) {
+  const int esz = (int)dtype_size(d->in_dtype);
+  memset(ga, 0, sizeof *ga);
+  ga->active = 1;
+  ga->rank = heap->rank;
+  ga->world = heap->world_size;
+  ga->heap_bases = heap->heap_bases;
+  ga->shard = gs.shard;
+  ga->ld_shard = gs.ld_shard;
+  ga->k_shard = gs.k_shard;
+  memset(p, 0, sizeof *p);
+  p->mode = tccl::kBgGatherCols;
+  p->slots = heap->world_size;  // every rank's shard, the own one included
+  p->rank = heap->rank;
+  p->world = heap->world_size;
+  p->heap_bases = heap->heap_bases;
+  p->block_rows = d->M;
+  p->pitch = (uint32_t)(d->lda * esz);
+  p->src_pitch = (uint32_t)(gs.ld_shard * esz);
+  p->upr = (uint32_t)((int64_t)gs.k_shard * esz / 16);
+  p->units = (uint32_t)d->M * p->upr;
+  p->pieces = (int)((p->units + tccl::kPieceUnits - 1) / tccl::kPieceUnits);
+  p->epoch = 1;
+  p->fault = c.fault;
+  p->spin_ticks = c.spin_ticks;
+}
+
+bool gather_in_place(const tccl_gemm_desc* d, const tccl_device_info& dev, int k_shard, int variant) {
+  if (variant == TCCL_S0_BULK || !use_macro(d, dev)) return false;
+  if (d->in_dtype != d->out_dtype || (d->in_dtype != TCCL_F16 && d->in_dtype != TCCL_BF16)) return false;
+  return k_shard % 64 == 0 && d->column_shards <= 1;
+}
+
 // GEMM (+ optional communication role) for one of the three operations.
 int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc* sync, const tccl_transport_desc* tr,
-                int variant, const tccl_device_info& dev, const tccl::GemmArgs& g, hipStream_t stream) {
+                int variant, const tccl_device_info& dev, const tccl::GemmArgs& g, hipStream_t stream,
+                const GatherSpec* gather = nullptr, const tccl_heap_view* heap = nullptr) {
   const int span = c.op != tccl::kOpNone ? check_comm_span(c) : 0;
   if (span) return span;
   const int total_tiles = g.tile_rows * g.tile_cols;
@@ -575,7 +631,10 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     // pulls (and, for a reduce-scatter, the reductions).
     if (build_push(c, g, &f.push)) c.directions &= ~tccl::kDirPush;
     memset(&f.reduce, 0, sizeof f.reduce);
-    if (build_reduce(c, sync, d->flags, &f.reduce, &f.m)) {
+    memset(&f.gather, 0, sizeof f.gather);
+    if (gather) {
+      build_gather_background(d, *gather, heap, c, &f.pull, &f.gather);
+    } else if (build_reduce(c, sync, d->flags, &f.reduce, &f.m)) {
       c.op = tccl::kOpNone;
       memset(&f.pull, 0, sizeof f.pull);
     } else if (build_background(c, &f.pull)) {
@@ -1034,8 +1093,9 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
   return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
 }
 
-int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,
-                         const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, void* stream) {
+static int allscatter_impl(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,
+                           const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, const GatherSpec* gather,
+                           hipStream_t stream) {
   int rc = check_gemm(d);
   if (rc) return rc;
   if ((rc = check_heap(heap))) return rc;
@@ -1056,7 +1116,12 @@ int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, c
   c.dst_ld = sc->dst_ld;
   c.dst_col_off = sc->dst_col_offset;
   if ((rc = set_task_units(&c, tr, false))) return rc;
-  return run_variant(d, c, sync, tr, variant, dev, g, (hipStream_t)stream);
+  return run_variant(d, c, sync, tr, variant, dev, g, stream, gather, heap);
+}
+
+int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,
+                         const tccl_sync_desc* sync, const tccl_transport_desc* tr, int32_t variant, void* stream) {
+  return allscatter_impl(d, sc, heap, sync, tr, variant, nullptr, (hipStream_t)stream);
 }
 
 int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* d, const void* shard, int64_t ld_shard, int32_t k_shard,
@@ -1068,16 +1133,28 @@ int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* d, const void* shard, int64_t 
   if (k_shard <= 0 || (int64_t)k_shard * heap->world_size != d->K)
     return fail(TCCL_ERR_INVALID, "chained: input_shard columns (%d) * world_size (%d) != W rows (%d)", k_shard,
                 heap->world_size, d->K);
-  // Stage 1: the gathered input (gemm->A) is filled from every rank's shard.
-  if ((rc = tccl_gather_cols((void*)d->A, d->lda, shard, ld_shard, d->M, k_shard, (int32_t)dtype_size(d->in_dtype), heap, tr, stream)))
-    return rc;
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
   // Stages 2 and 3: the GEMM, whose whole output goes to every peer's output.
   tccl_scatter_desc sc;
   sc.src_col_offset = 0;
   sc.cols = d->N;
   sc.dst_ld = (int32_t)d->ldc;
   sc.dst_col_offset = 0;
-  return tccl_gemm_allscatter(d, &sc, heap, sync, tr, variant, stream);
+  const int esz = (int)dtype_size(d->in_dtype);
+  const bool shard_ok = shard && ld_shard >= k_shard && (ld_shard * esz) % 16 == 0 && ((int64_t)k_shard * esz) % 16 == 0 &&
+                        aligned16(shard) && (255 * ld_shard + k_shard) * (int64_t)esz <= 0xffffffffll;
+  if (shard_ok && gather_in_place(d, dev, k_shard, variant)) {
+    // One launch: the K loops read every rank's shard where it lies, and the gathered
+    // workspace (gemm->A) is filled on the side while they run.
+    if ((rc = check_rows_span(d->M, (d->lda > ld_shard ? d->lda : ld_shard) * esz))) return rc;
+    const GatherSpec gs{shard, ld_shard, k_shard};
+    return allscatter_impl(d, &sc, heap, sync, tr, variant, &gs, (hipStream_t)stream);
+  }
+  // Stage 1 as a launch of its own: the gathered input (gemm->A) is filled from every rank's shard.
+  if ((rc = tccl_gather_cols((void*)d->A, d->lda, shard, ld_shard, d->M, k_shard, (int32_t)esz, heap, tr, stream)))
+    return rc;
+  return allscatter_impl(d, &sc, heap, sync, tr, variant, nullptr, (hipStream_t)stream);
 }
 
 int tccl_gemm_allgather(const tccl_gemm_desc* d, void* out, int64_t ld_out, const tccl_heap_view* heap,

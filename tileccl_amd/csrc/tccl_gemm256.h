@@ -126,7 +126,7 @@ struct ReduceArgs {
 // counter fetches which are themselves left in flight for one K step.  What the K loops did
 // not get to is finished after the last tile, with bounded waits.  Groups must cover the rows
 // in ascending order (build_tile_group_plan emits them so: tileccl_v2/tile_group.py:244-301).
-enum BackgroundMode { kBgNone = 0, kBgGather = 1 };
+enum BackgroundMode { kBgNone = 0, kBgGather = 1, kBgGatherCols = 2 };
 struct PullArgs {
   int mode;
   int slots;                   // blocks to process: the peers
@@ -149,6 +149,22 @@ struct PullArgs {
   int64_t* fault;
   int64_t spin_ticks;
   int64_t word_stride;         // as in CommArgs: 0 = a peer's counters sit in its heap slice
+  uint32_t src_pitch;          // kBgGatherCols: bytes per row of a shard (`pitch` is the workspace's)
+};
+// Gathered input read in place (the gather stage of ChainedAGGemmRSPattern folded into the
+// GEMM, patterns/chained_ag_gemm_rs.py:262-391): the GEMM's A operand is the concatenation
+// along K of every rank's (M x k_shard) shard, and shard p sits at the same offset of slice
+// p.  The K loop fetches its A stages straight from the shard that holds the K range, so it
+// does not depend on the gathered workspace; that workspace (GemmArgs::A) is still filled, by
+// the background transfer (mode kBgGatherCols: every rank's shard, the own one included, is
+// copied into its column block while the K loops run).  k_shard is a multiple of the K step.
+struct GatherArgs {
+  int active;
+  int rank, world;
+  const int64_t* heap_bases;
+  const void* shard;   // this rank's shard; a peer's sits at the same slice offset
+  int64_t ld_shard;    // elements
+  int k_shard;         // columns per shard
 };
 constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter word per wavefront (64 lanes x 4 B)
 // Of a SIMD's two wavefronts the older one (wavefronts 0..3 of the workgroup) wins the matrix
@@ -207,7 +223,7 @@ TCCL_D void warm_kernargs() {
   asm volatile("" ::"s"(any));
 }
 
-template <typename InT, typename OutT, bool kWithReduce = false>
+template <typename InT, typename OutT, bool kWithReduce = false, bool kGatherA = false>
 struct Gemm256 {
   typedef typename Mfma<InT>::Vec Vec;
   static constexpr int kEszIn = sizeof(InT);
@@ -225,6 +241,7 @@ struct Gemm256 {
   const int pull_offset;
   const int push_offset;    // byte offset of a PushArgs in the kernel arguments; < 0: no push
   const int reduce_offset;  // byte offset of a ReduceArgs in the kernel arguments; < 0: none
+  const int gather_offset;  // byte offset of a GatherArgs in the kernel arguments (kGatherA only)
   // The two pipeline stages are two separate __shared__ arrays: loads that write LDS directly
   // are tracked per LDS variable, so a read of one stage need not wait for a load into the other.
   char* lds;   // stage 0 (also the epilogue's staging area)
@@ -238,8 +255,8 @@ struct Gemm256 {
   }
 
   TCCL_D Gemm256(const GemmArgs& args, int pull_args_offset, int push_args_offset, int reduce_args_offset, char* stage0,
-                 char* stage1, char* landing_words)
-      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+                 char* stage1, char* landing_words, int gather_args_offset = -1)
+      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), gather_offset(gather_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
         wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
@@ -258,7 +275,30 @@ struct Gemm256 {
     __amdgpu_buffer_rsrc_t a, b;
     uint32_t off_a[4], off_b[4];
     uint32_t step_a, step_b;
+    // kGatherA: `a` is the window onto the shard that holds K steps [kt_base, kt_switch)
+    int kt_base, kt_switch, row0;
   };
+  typedef const __attribute__((address_space(4))) GatherArgs* GatherPtr;
+
+  // Point `s.a` at the shard that holds K step kt (kGatherA).  Steps past K stay on the last
+  // shard: their chunks are redirected past the end of the window by issue_a and read as zero.
+  TCCL_D void select_shard(Source& s, int kt) const {
+    const GatherPtr ga = late_kernarg_ptr<GatherArgs>(gather_offset);
+    const int per_shard = ga->k_shard / kStepK;
+    int p = kt / per_shard;
+    if (p >= ga->world) p = ga->world - 1;
+    const int64_t base = (int64_t)(uintptr_t)ga->shard + (table(ga->heap_bases, p) - table(ga->heap_bases, ga->rank)) +
+                         (int64_t)s.row0 * ga->ld_shard * kEszIn;
+    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)(uintptr_t)base, 0,
+                                            clamp_u32(((int64_t)(g.M - 1 - s.row0) * ga->ld_shard + ga->k_shard) * kEszIn), 0x00020000);
+    s.kt_base = p * per_shard;
+    s.kt_switch = p + 1 < ga->world ? (p + 1) * per_shard : 0x7fffffff;
+  }
+  // Before the loads of K step kt are issued.
+  TCCL_D void follow_shards(Source& s, int kt) const {
+    if constexpr (kGatherA)
+      if (kt >= s.kt_switch) select_shard(s, kt);
+  }
 
   static TCCL_D uint32_t clamp_u32(int64_t v) { return v > 0xffffffffll ? 0xffffffffu : (v < 0 ? 0u : (uint32_t)v); }
 
@@ -274,7 +314,9 @@ struct Gemm256 {
     for (int i = 0; i < 4; ++i) {
       const int row = 8 * (4 * wave + i) + (lane >> 3);
       const int kc = (lane & 7) ^ ((row >> 1) & 7);
-      s.off_a[i] = (uint32_t)(row * g.lda * kEsz + kc * 16);
+      int64_t lda = g.lda;
+      if constexpr (kGatherA) lda = late_kernarg_ptr<GatherArgs>(gather_offset)->ld_shard;
+      s.off_a[i] = (uint32_t)(row * lda * kEsz + kc * 16);
       if constexpr (kFp8) {
         const int k = 4 * (4 * wave + i) + (lane >> 4);
         const int c = (lane & 15) ^ (2 * (k & 7));
@@ -287,6 +329,10 @@ struct Gemm256 {
     }
     s.step_a = kStepK * kEsz;
     s.step_b = (uint32_t)(kStepK * g.ldb * kEsz);
+    s.kt_base = 0;
+    s.kt_switch = 0x7fffffff;
+    s.row0 = row0;
+    if constexpr (kGatherA) select_shard(s, 0);
     return s;
   }
 
@@ -295,7 +341,7 @@ struct Gemm256 {
   TCCL_D void issue_a(char* stage, const Source& s, int kt, int i) const {
     const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);  // as in make_source
     const bool dead = kt * kStepK + kc * kChunkK >= g.K;
-    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + kt * s.step_a;
+    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + (kGatherA ? kt - s.kt_base : kt) * s.step_a;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + 8 * (4 * wave + i) * kARow256), 16, oa, 0, 0, 0);
   }
   TCCL_D void issue_b(char* stage, const Source& s, int kt, int i) const {
@@ -540,6 +586,16 @@ struct Gemm256 {
     st.ready_units = 0;
     st.probe_group = -1;
     st.backoff = 0;
+    if constexpr (kGatherA) {
+      // Block `slot` = rank `slot`'s shard (resident input: nothing to wait for) into column
+      // block `slot` of the gathered workspace.
+      const GatherPtr ga = late_kernarg_ptr<GatherArgs>(gather_offset);
+      st.src_base = (int64_t)(uintptr_t)ga->shard + (table(ga->heap_bases, slot) - table(ga->heap_bases, ga->rank));
+      st.dst_base = (int64_t)(uintptr_t)g.A + (int64_t)slot * ga->k_shard * kEszIn;
+      st.ready_units = a->units;
+      st.gidx = a->n_groups;
+      return;
+    }
     const int64_t mine = table(a->heap_bases, a->rank);
     const int peer = slot < a->rank ? slot : slot + 1;
     const int64_t theirs = table(a->heap_bases, peer);
@@ -645,7 +701,9 @@ struct Gemm256 {
       for (int j = 0; j < kPullLoads; ++j) {
         const bool valid = first + (uint32_t)(64 * j + lane) < st.units;
         const uint32_t off = valid ? st.row[j] * st.pitch + st.col[j] * 16u : 0u;  // idle lanes touch the block's first unit
-        st.piece[slot][j] = ld16<kCoherent>(src, off);
+        uint32_t from = off;
+        if constexpr (kGatherA) from = valid ? st.row[j] * a->src_pitch + st.col[j] * 16u : 0u;
+        st.piece[slot][j] = ld16<kCoherent>(src, from);
         st.pend_off[slot][j] = valid ? off : kNoUnit;
       }
       st.pend_mask |= 1 << slot;
@@ -732,7 +790,7 @@ struct Gemm256 {
               uint32_t row, col;
               pull_unit(a, lp, j, valid, row, col);
               const uint32_t o = row * a->pitch + col * 16u;
-              v[k][j] = ld16<kCoherent>(src, o);
+              v[k][j] = ld16<kCoherent>(src, kGatherA ? row * a->src_pitch + col * 16u : o);
               off[k][j] = valid ? o : kNoUnit;
             }
             loaded[k] = true;
@@ -1075,7 +1133,7 @@ struct Gemm256 {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const Source src = make_source(row0, col0);
+    Source src = make_source(row0, col0);
     const Reader rd = make_reader();
     // K steps are taken in pairs so that each call names its two stages statically and the
     // accumulators flow through one straight loop body.  An odd step count is rounded up: the
@@ -1100,7 +1158,9 @@ struct Gemm256 {
       f.fb[0][1] = load_b8(lds, rd, 0, 1);
       f.ring[0] = load_a8(lds, rd, 0, 0);
       for (int kt = 0; kt < ksteps; kt += 2) {
+        follow_shards(src, kt + 1);
         k_step8(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
+        follow_shards(src, kt + 2);
         k_step8(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
     } else {
@@ -1109,7 +1169,9 @@ struct Gemm256 {
       f.ring[0] = load_a16(lds, rd, 0, 0);
       f.ring[1] = load_a16(lds, rd, 0, 1);
       for (int kt = 0; kt < ksteps; kt += 2) {
+        follow_shards(src, kt + 1);
         k_step16(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
+        follow_shards(src, kt + 2);
         k_step16(lds1, lds, src, rd, kt + 2, acc, f, pull, 1);
       }
       pull_retire(pull, pa(), bgw, 1);  // the last step's piece: nothing is carried through the epilogue
