@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from tileccl_amd.patterns.contracts import resolve_pattern_execution
-from tileccl_amd.patterns.runtime import resolve_dual_role_scheduler, resolve_stage_role_scheduler
+from tileccl_amd.patterns.runtime import resolve_dual_role_scheduler
 
 
 def T(rows, cols):
@@ -93,35 +93,16 @@ def test_dual_role_scheduler():
     assert (s.compute_sms, s.comm_sms) == (1, 1)
     s = resolve_dual_role_scheduler(256, compute_sms=200, comm_sms=40)
     assert (s.compute_sms, s.comm_sms, s.policy) == (200, 40, "explicit")
+    assert s.to_dict() == {"total_sms": 256, "compute_sms": 200, "comm_sms": 40, "policy": "explicit"}
+    assert resolve_dual_role_scheduler(3, comm_sm_fraction=0.0).comm_sms == 1  # never fewer than one mover
+    with pytest.raises(ValueError, match="requires both compute_sms and comm_sms to be > 0"):
+        resolve_dual_role_scheduler(256, comm_sms=8)
     with pytest.raises(ValueError, match="requires at least 2 compute units"):
         resolve_dual_role_scheduler(1)
     with pytest.raises(ValueError, match="requires both compute_sms and comm_sms to be > 0"):
         resolve_dual_role_scheduler(256, compute_sms=10)
     with pytest.raises(ValueError, match=r"cannot exceed the device SM count: 200 \+ 100 > 256"):
         resolve_dual_role_scheduler(256, compute_sms=200, comm_sms=100)
-
-
-def test_stage_role_scheduler():
-    """Hand-computed from the reference's rule: budget = max(2, int(total * 0.2)), halved
-    (gather gets the floor), compute takes the rest (runtime.py:232-291)."""
-    s = resolve_stage_role_scheduler(256)
-    assert (s.gather_sms, s.compute_sms, s.scatter_sms, s.policy) == (25, 205, 26, "fractional_split")
-    assert s.collective_sms == 51 and s.grid_sms == 256
-    s = resolve_stage_role_scheduler(132)  # int(26.4) = 26 -> 13 + 13
-    assert (s.gather_sms, s.compute_sms, s.scatter_sms) == (13, 106, 13)
-    s = resolve_stage_role_scheduler(3)  # budget max(2, 0) = 2 -> 1 + 1, one CU computes
-    assert (s.gather_sms, s.compute_sms, s.scatter_sms) == (1, 1, 1)
-    s = resolve_stage_role_scheduler(10, collective_sm_fraction=0.99)  # budget capped at total - 1
-    assert (s.gather_sms, s.compute_sms, s.scatter_sms) == (4, 1, 5)
-    s = resolve_stage_role_scheduler(256, gather_sms=16, compute_sms=200, scatter_sms=32)
-    assert (s.gather_sms, s.compute_sms, s.scatter_sms, s.policy) == (16, 200, 32, "explicit")
-    assert s.to_dict()["grid_sms"] == 248
-    with pytest.raises(ValueError, match="requires at least 3 compute units, got total_sms=2"):
-        resolve_stage_role_scheduler(2)
-    with pytest.raises(ValueError, match="requires gather_sms, compute_sms, and scatter_sms to be > 0"):
-        resolve_stage_role_scheduler(256, gather_sms=16)
-    with pytest.raises(ValueError, match=r"cannot exceed the device SM count: 100 \+ 100 \+ 100 > 256"):
-        resolve_stage_role_scheduler(256, gather_sms=100, compute_sms=100, scatter_sms=100)
 
 
 # ---- public op contract, exercised with a stand-in context on CPU tensors ---------------------------------

@@ -107,8 +107,6 @@ def test_argument_errors(lib):
         W2 = ctxs[0].zeros(128, 128, dtype=torch.float16)
         with pytest.raises(ValueError, match="input_shard must live in the symmetric heap"):
             ChainedAGGemmRSPattern(ctxs[0]).execute(off_heap, W2, out)
-        roles = ChainedAGGemmRSPattern(ctxs[0]).stage_roles()
-        assert roles.gather_sms + roles.compute_sms + roles.scatter_sms <= roles.total_sms
     finally:
         for c in ctxs:
             c.heap.cleanup()

@@ -5,12 +5,15 @@ every rank holds an ``(M, K_shard)`` column shard of the input; the pattern gath
 shards into an ``(M, K)`` workspace (column block ``p`` from rank ``p``), multiplies by the full
 weight ``W (K, N)`` and stores the ``(M, N)`` result into every peer's output as well as its own.
 
-Stages on MI355X: the gather is one bulk copy launch (an HBM-bound scan that the GEMM's
-first tiles would have to wait for anyway: the large-tile GEMM fills every CU, so no gather
-workgroup could run beside it); the GEMM and the stores to the peers overlap according to
-``schedule``: ``"bulk_sync"`` (GEMM kernel, then a copy kernel), ``"wg_specialized"`` (one
-launch, per-tile) or ``"tile_group"`` (one launch, per TileGroup; the default).  With the
-256 x 256 tile the stores leave from the GEMM epilogue.
+Stages on MI355X, by ``schedule``: ``"bulk_sync"`` is three launches (gather copy, GEMM
+kernel, copy to the peers).  ``"wg_specialized"`` (per tile) and ``"tile_group"`` (per
+TileGroup; the default) are one launch on the 256 x 256 tile: the K loops read every
+rank's shard where it lies (the shards are resident inputs at the same offset of every
+slice), the gathered workspace is filled on the side by the same launch's background
+transfer, and the stores to the peers leave from the GEMM epilogue, so neither the gather
+nor the scatter is waited for.  Shapes the large tile does not take (small outputs, shards
+that are not whole 64-element K steps) run the gather as a bulk launch ahead of the fused
+GEMM + scatter launch.
 
 The reference kernel addresses the workspace rows with the column stride
 (``gathered_ptr + offs_m * stride_gk``, :298 and :353), so its rows overlap; the result
@@ -26,7 +29,6 @@ import torch
 
 from tileccl_amd import _launch, _lib
 from tileccl_amd.patterns.hip_patterns import BulkSyncPattern, TileGroupPattern, WGSpecializedPattern
-from tileccl_amd.patterns.runtime import resolve_stage_role_scheduler
 
 _SCHEDULES = {"bulk_sync": BulkSyncPattern, "wg_specialized": WGSpecializedPattern, "tile_group": TileGroupPattern}
 
@@ -34,10 +36,9 @@ _SCHEDULES = {"bulk_sync": BulkSyncPattern, "wg_specialized": WGSpecializedPatte
 class ChainedAGGemmRSPattern:
     """Three stages, gather -> GEMM -> scatter, for column-sharded inputs.
 
-    Arguments as in the reference (:40-75).  The ``*_SMS`` arguments are validated and
-    resolved with the reference's stage-role policy and reported by ``stage_roles()``; the
-    launch geometry itself follows the library defaults, because the stages are not
-    co-resident roles here (see the module docstring).
+    Arguments as in the reference (:40-75).  The ``*_SMS`` arguments are accepted for
+    signature parity; the launch geometry follows the library defaults, because the stages
+    are not separate workgroup roles here (see the module docstring).
     """
 
     name: str = "chained_ag_gemm_rs"
@@ -62,15 +63,6 @@ class ChainedAGGemmRSPattern:
         # The GEMM + scatter stages reuse the all-scatter pattern's plan and signal words.
         self._stage = _SCHEDULES[schedule](ctx, BLOCK_M=BLOCK_M, BLOCK_N=BLOCK_N, BLOCK_K=BLOCK_K)
         self._last_sync: _launch.SyncWords | None = None
-
-    def stage_roles(self):
-        """The reference's gather / compute / scatter split for this device (:77-85)."""
-        return resolve_stage_role_scheduler(
-            self.ctx.backend.get_device_properties().compute_units,
-            gather_sms=self.GATHER_SMS,
-            compute_sms=self.COMPUTE_SMS,
-            scatter_sms=self.SCATTER_SMS,
-        )
 
     def execute(
         self,

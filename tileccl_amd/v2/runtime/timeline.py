@@ -195,15 +195,11 @@ class TimelineRecorder:
                             lane_order=lane_order)
 
 
-_CATEGORY_COLORS = {
-    "producer": "#4c78a8", "ingress": "#b279a2", "frontier": "#f58518", "compute": "#54a24b",
-    "aggregation": "#e45756", "marker": "#333333", "span": "#72b7b2",
-}
-
-
 def render_timeline_png(events: Sequence[TimelineEvent], path: Path, *, title: str,
                         lane_order: Sequence[str] | None = None) -> None:
-    """One horizontal lane per ``event.lane``; spans as bars, zero-length events as ticks."""
+    """A Gantt chart: one row per lane (first lane on top), one bar per span, a thin mark
+    per zero-length event.  Categories share a colour taken from matplotlib's ``tab10``
+    cycle in order of first appearance; an event's own ``color`` wins."""
     if not events:
         raise ValueError("Cannot render an empty timeline")
     import matplotlib
@@ -212,24 +208,26 @@ def render_timeline_png(events: Sequence[TimelineEvent], path: Path, *, title: s
     import matplotlib.pyplot as plt
 
     lanes = _lanes_in_order(events, lane_order)
-    row = {lane: len(lanes) - i for i, lane in enumerate(lanes)}
-    t_max = max(e.end_ms for e in events)
-    fig, ax = plt.subplots(figsize=(12, max(2.8, 0.55 * len(lanes) + 1.6)))
+    palette = plt.get_cmap("tab10").colors
+    shade: dict[str, object] = {}
     for e in events:
-        y, color = row[e.lane], e.color or _CATEGORY_COLORS.get(e.category, _CATEGORY_COLORS["span"])
-        if e.duration_ms == 0:
-            ax.vlines(e.start_ms, y - 0.23, y + 0.23, color=color, linewidth=1.5)
-            continue
-        ax.barh(y, e.duration_ms, left=e.start_ms, height=0.36, color=color, edgecolor="white")
-        if e.duration_ms >= max(0.08, t_max * 0.035):
-            ax.text(e.start_ms + e.duration_ms / 2, y, e.label or e.name, fontsize=8, ha="center", va="center", color="white")
-    ax.set_title(title)
-    ax.set_yticks([row[lane] for lane in lanes])
-    ax.set_yticklabels(lanes)
-    ax.set_xlabel("Elapsed time (ms)")
-    ax.set_xlim(0, t_max * 1.06 if t_max > 0 else 1.0)
-    ax.grid(axis="x", alpha=0.5)
-    fig.tight_layout()
+        shade.setdefault(e.category, palette[len(shade) % len(palette)])
+    horizon = max(e.end_ms for e in events) or 1.0
+    mark = horizon / 400.0  # width given to instantaneous events so that they stay visible
+    fig, ax = plt.subplots(figsize=(11, 1.2 + 0.5 * len(lanes)), constrained_layout=True)
+    for row, lane in enumerate(lanes):
+        mine = [e for e in events if e.lane == lane]
+        ax.broken_barh([(e.start_ms, e.duration_ms or mark) for e in mine], (row - 0.3, 0.6),
+                       facecolors=[e.color or shade[e.category] for e in mine])
+        for e in mine:
+            text = e.label or e.name
+            if e.duration_ms / horizon * 11 * 72 > 5.5 * len(text):  # the bar is wider than the text at 7 pt
+                ax.annotate(text, (e.start_ms + e.duration_ms / 2, row), ha="center", va="center", fontsize=7)
+    ax.set(title=title, xlabel="Elapsed time (ms)", xlim=(0, horizon * 1.02), ylim=(len(lanes) - 0.5, -0.5))
+    ax.set_yticks(range(len(lanes)), labels=lanes)
+    ax.xaxis.grid(True, linewidth=0.4)
+    ax.legend(handles=[plt.Rectangle((0, 0), 1, 1, color=c) for c in shade.values()], labels=list(shade),
+              loc="upper right", fontsize=7, ncols=min(len(shade), 4), frameon=False)
     path.parent.mkdir(parents=True, exist_ok=True)
-    fig.savefig(path, dpi=160)
+    fig.savefig(path, dpi=150)
     plt.close(fig)
