@@ -429,8 +429,17 @@ int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
 // after the last tile then does it).
 bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   memset(p, 0, sizeof *p);
-  if (c.op != tccl::kOpAllGather || c.granularity != tccl::kPerGroup || !(c.directions & tccl::kDirPull) || c.world <= 1) return false;
-  if (!c.row_ends || !c.tile_counts || !c.counter) return false;
+  if (c.op != tccl::kOpAllGather || c.granularity == tccl::kBulk || !(c.directions & tccl::kDirPull) || c.world <= 1) return false;
+  const bool by_tile = c.granularity == tccl::kPerTile;
+  int band_shift = 0;
+  if (by_tile) {
+    // One probe looks at the locks of two plan-tile rows, 32 lanes each; the lock index needs
+    // the swizzle band as a shift.
+    while ((1 << band_shift) < c.group_m) ++band_shift;
+    if (!c.locks || c.tile_cols > 32 || (1 << band_shift) != c.group_m) return false;
+  } else if (!c.row_ends || !c.tile_counts || !c.counter) {
+    return false;
+  }
   const int64_t row_bytes = (int64_t)c.N * c.esize;
   const int64_t block_bytes = (int64_t)c.M * c.ld_out_bytes;
   if (row_bytes % 16 || c.ld_out_bytes % 16 || block_bytes >= (int64_t)1 << 32) return false;
@@ -446,10 +455,12 @@ bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   p->upr = (uint32_t)(row_bytes / 16);
   p->units = (uint32_t)p->block_rows * p->upr;
   p->pieces = (int)((p->units + tccl::kPieceUnits - 1) / tccl::kPieceUnits);
-  p->counter = c.counter;
+  p->counter = by_tile ? c.locks : c.counter;
   p->row_ends = c.row_ends;
   p->tile_counts = c.tile_counts;
-  p->n_groups = c.n_groups;
+  p->n_groups = by_tile ? (c.tile_rows + 1) / 2 : c.n_groups;
+  p->tile_mode = by_tile ? 1 : 0;
+  p->group_m_shift = band_shift;
   p->epoch = c.epoch;
   p->barrier = c.barrier;
   p->trace_done_clock = c.trace_done_clock;
