@@ -553,6 +553,16 @@ int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
 // reductions of the reduce-scatter configurations (4 per CU ahead of 8 by 3-4 %).
 int bulk_comm_wgs(const tccl_device_info& dev) { return dev.compute_units * 4; }
 
+// The second kernel of S0 waits for nothing, so a plan's TileGroups mean nothing to it: it
+// sweeps the whole block (a reduce-scatter: each owner's shard) as one run of tasks.  Cut
+// along the plan's groups, its tasks came out ragged at every group border (8192 x 4096
+// all-gather: 123 us with eight groups against 117 us with one).
+void make_bulk(tccl::CommArgs* c) {
+  c->granularity = tccl::kBulk;
+  c->row_starts = c->row_ends = c->tile_counts = nullptr;
+  c->n_groups = c->op == tccl::kOpReduceScatter ? c->world : 1;
+}
+
 // The shards that make up the GEMM's A operand, when the chained operation reads them in place.
 struct GatherSpec {
   const void* shard;
@@ -616,7 +626,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     if (variant == TCCL_S0_BULK) {
       int rc = launch_gemm256(d->in_dtype, d->out_dtype, g, m, wgs, stream);
       if (rc) return rc;
-      c.granularity = tccl::kBulk;
+      make_bulk(&c);
       if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
       return launch_comm(c, bulk_comm_wgs(dev), stream);
     }
@@ -660,7 +670,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     memset(&none, 0, sizeof none);
     int rc = launch_fused(d->in_dtype, d->out_dtype, g, s, none, compute, 0, trace_start, stream);
     if (rc) return rc;
-    c.granularity = tccl::kBulk;
+    make_bulk(&c);
     if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
     return launch_comm(c, bulk_comm_wgs(dev), stream);
   }
