@@ -903,12 +903,12 @@ struct Gemm256 {
   //
   // The step's one barrier sits before item 14, not at the end.  There this wave has issued
   // (and, after the lgkmcnt wait, finished) its last read of `cur`, and its loads into `nxt`,
-  // issued during items 0..6, have landed; behind the barrier items 14 and 15 already fetch
+  // issued during items 0..7, have landed; behind the barrier items 14 and 15 already fetch
   // the next step's first operands from `nxt`, so the matrix pipe does not drain while the
   // first LDS reads of a step are in flight.  Measured against a barrier at the end of the
   // step (4096^3 fp16): 128.4 us instead of 133.6.
   //
-  // The loads go out in pairs at items 0, 2, 4, 6.  Issuing a load holds the wave for as long
+  // The loads go out one per item over items 0..7.  Issuing a load holds the wave for as long
   // as the address unit takes to accept it (about 16 clocks per KiB instruction, four times
   // that when the four SIMDs' waves issue in the same item), and nothing else of the wave
   // issues meanwhile; later or denser placements measured slower.
