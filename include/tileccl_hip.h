@@ -248,6 +248,26 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
                      const tccl_heap_view* heap, const tccl_transport_desc* transport,
                      int32_t emulate_peer, void* stream);
 
+/* tccl_allreduce_staged: the staged peer-read all-reduce of the public allreduce launcher
+ * (_allreduce_staged_kernel / _allreduce_staged_kernel_ws2, primitives/collectives.py:840-1044;
+ * launcher :1882-1946, workspace :2813-2838).  In place on `tensor` (numel elements of `dtype`
+ * F16 / BF16 / F32, whole 16-byte units) at the same offset of every rank's slice.  Per chunk of
+ * chunk_elems a rank snapshots its values into its `staging` slot, publishes epoch
+ * base_epoch + chunk in `published[slot]`, waits for every peer's matching epoch, adds the
+ * ranks' values in ascending rank order (fp32 accumulation, one rounding: every rank stores the
+ * same bits; the reference starts from its own values and adds in the tensor's type) and
+ * acknowledges in the peer's `consumed[slot]`; a rank leaves a slot once world - 1 peers have
+ * acknowledged.  staging (slots x chunk_elems), published and consumed
+ * (int32[slots], zero before the first call) live in the heap.  `ranks` is the bit mask of the
+ * ranks whose roles this launch carries: one process per GPU passes 1 << rank; on one GPU, where
+ * the ranks are slices of one arena, all of them run as workgroups of one launch (slots
+ * workgroups per rank, all resident).  The caller advances base_epoch by the chunk count per
+ * call.  `fault` / `spin_limit_ns` as in tccl_sync_desc. */
+int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* staging, int32_t* published,
+                          int32_t* consumed, int32_t chunk_elems, int32_t slots, int32_t base_epoch,
+                          uint32_t ranks, const tccl_heap_view* heap, int64_t* fault, int64_t spin_limit_ns,
+                          void* stream);
+
 /* ---- fused operations --------------------------------------------------------------------
  * variant S0: GEMM kernel, then the communication kernel, stream-ordered.
  * variant S1: one launch; GEMM workgroups signal locks[tile]; communication workgroups

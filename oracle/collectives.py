@@ -166,6 +166,18 @@ def allreduce(tensors):
     return [full.clone() for _ in tensors]
 
 
+def allreduce_staged(tensors):
+    """Every rank's tensor after the staged all-reduce (the protocol of _allreduce_staged_kernel,
+    /root/reference/tileccl/primitives/collectives.py:840-962): the ranks' values added in
+    ascending rank order in fp32 and rounded once, the same bits on every rank.  (The reference
+    kernel adds in the tensor dtype starting from the rank's own values; for two ranks, and for
+    values whose sums are exact, the two agree.)"""
+    acc = tensors[0].float()
+    for t in tensors[1:]:
+        acc = acc + t.float()
+    return [acc.to(tensors[0].dtype) for _ in tensors]
+
+
 def expected_counters(tile_counts, epoch: int = 1):
     """counter[g] after ``epoch`` launches without reset: every tile of the group signalled once each."""
     return [epoch * t for t in tile_counts]

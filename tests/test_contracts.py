@@ -196,3 +196,25 @@ def test_support_matrix_shape():
     assert sorted(m["collectives"]) == ["allgather", "allreduce", "broadcast", "reduce_scatter", "scatter"]
     assert m["collectives"]["allreduce"]["state"] == "partial"  # needs a heap, like the ops
     assert m["execution_paths"]["tile_group"] == {"state": "supported", "detail": "one launch, per-TileGroup counters"}
+
+
+def test_staged_allreduce_execution_policy():
+    """Chunk and slot choice of the staged all-reduce: host arithmetic only."""
+    from tileccl_amd.primitives.collectives import resolve_staged_execution as resolve
+
+    # 1 MiB fp16 on two ranks: 64 chunks of 16 KiB, a slot each
+    assert resolve(1 << 19, 2, 2) == (8192, 64, 64)
+    # 16 MiB: the slots (256) no longer outnumber 16 KiB chunks -> 64 KiB chunks, every slot used once
+    assert resolve(1 << 23, 2, 2) == (32768, 256, 256)
+    # eight ranks: 128 slots each stay resident
+    assert resolve(1 << 26, 2, 8) == (32768, 2048, 128)
+    # a tensor smaller than a chunk: one chunk of its own size, rounded up to whole units
+    assert resolve(24, 2, 2) == (24, 1, 1)
+    assert resolve(8, 4, 3) == (8, 1, 1)
+    # explicit values are kept; slots never exceed the chunks
+    assert resolve(10000, 2, 2, chunk_elems=4096, pipeline_slots=8) == (4096, 3, 3)
+    import pytest
+    with pytest.raises(ValueError, match="multiple of 8"):
+        resolve(4096, 2, 2, chunk_elems=100)
+    with pytest.raises(ValueError, match="at least 1"):
+        resolve(4096, 2, 2, pipeline_slots=0)

@@ -158,6 +158,100 @@ def test_allreduce_in_place_any_call_order(lib, world, numel, dtype):
         close(heaps)
 
 
+@pytest.mark.parametrize("world,numel,dtype,chunk,slots", [
+    (2, 1 << 16, torch.float16, None, None),      # two chunks of 64 KiB, a slot each
+    (2, 1 << 20, torch.bfloat16, 4096, 4),        # 256 chunks through 4 slots: every slot reused 64 times
+    (3, 40 * 8, torch.float16, 64, 2),            # ragged: five chunks, the last one short, odd count over two slots
+    (4, 1 << 18, torch.float32, None, None),
+    (8, 3 * 4096 + 8, torch.float16, 4096, None), # last chunk of one unit
+    (2, 8, torch.float16, None, None),            # one 16-byte unit
+])
+def test_staged_allreduce_all_roles_in_one_launch(lib, world, numel, dtype, chunk, slots):
+    """Bit-exact against the oracle on every rank, on two calls in a row over the same workspace
+    (the second with the first's results as input: epochs continue, slots are reused)."""
+    from tileccl_amd.primitives import allreduce_staged
+
+    heaps = heaps_of(world)
+    try:
+        cpu = [seeded((numel,), 70 + r, dtype) for r in range(world)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        for _ in range(2):
+            want = oracle.allreduce_staged(cpu)
+            fault = allreduce_staged(ts, heaps, chunk_elems=chunk, pipeline_slots=slots)
+            torch.cuda.synchronize()
+            assert int(fault.item()) == 0
+            for r in range(world):
+                assert torch.equal(bits(ts[r]).cpu(), bits(want[r])), r
+            cpu = [(w * 0.25).to(dtype) for w in want]  # keep the values in range for the second call
+            for t, c in zip(ts, cpu):
+                t.copy_(c)
+        if world == 2:  # two addends commute: the same bits as the reduce-scatter based all-reduce
+            assert torch.equal(bits(oracle.allreduce_staged(cpu)[0]), bits(oracle.allreduce(cpu)[0]))
+    finally:
+        close(heaps)
+
+
+def test_staged_allreduce_integer_valued_sums_are_exact(lib):
+    """A check that does not go through the oracle: small integers add exactly in every order and type."""
+    from tileccl_amd.primitives import allreduce_staged
+
+    world, numel = 4, 5 * 4096
+    heaps = heaps_of(world)
+    try:
+        g = torch.Generator().manual_seed(5)
+        cpu = [torch.randint(-60, 60, (numel,), generator=g).to(torch.float16) for _ in range(world)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        allreduce_staged(ts, heaps, chunk_elems=4096, pipeline_slots=3)
+        torch.cuda.synchronize()
+        total = sum(c.long() for c in cpu)
+        for t in ts:
+            assert torch.equal(t.cpu().long(), total)
+    finally:
+        close(heaps)
+
+
+def test_staged_allreduce_missing_role_times_out_and_reports(lib):
+    """Only rank 0's role is launched: its wait for rank 1's epoch runs into the (tiny) bound,
+    the fault word is raised, the kernel exits, and rank 0's tensor is left as it was."""
+    from tileccl_amd.primitives import allreduce_staged
+
+    heaps = heaps_of(2)
+    try:
+        cpu = [seeded((4096,), 90 + r, torch.float16) for r in range(2)]
+        ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+        fault = allreduce_staged(ts, heaps, ranks=(0,), spin_limit_ns=200_000)
+        torch.cuda.synchronize()
+        assert int(fault.item()) != 0
+        assert torch.equal(bits(ts[0]).cpu(), bits(cpu[0]))
+        assert torch.equal(bits(ts[1]).cpu(), bits(cpu[1]))
+    finally:
+        close(heaps)
+
+
+def test_staged_allreduce_contracts(lib):
+    from tileccl_amd.primitives import allreduce_staged
+
+    heaps = heaps_of(2)
+    try:
+        a = [h.allocate_tensor((64,), torch.float16) for h in heaps]
+        with pytest.raises(ValueError, match="Only op='sum'"):
+            allreduce_staged(a, heaps, op="max")
+        with pytest.raises(ValueError, match="one tensor and one heap per rank"):
+            allreduce_staged(a[:1], heaps)
+        with pytest.raises(ValueError, match="chunk_elems=12 must be a positive multiple of 8"):
+            allreduce_staged(a, heaps, chunk_elems=12)
+        extra = heaps[1].allocate_tensor((64,), torch.float16)  # rank 1's heap is now one allocation ahead
+        b = [heaps[0].allocate_tensor((64,), torch.float16), heaps[1].allocate_tensor((64,), torch.float16)]
+        with pytest.raises(ValueError, match="same heap offset"):
+            allreduce_staged(b, heaps)
+        del extra
+        ints = [h.allocate_tensor((64,), torch.int32) for h in heaps]
+        with pytest.raises(ValueError):
+            allreduce_staged(ints, heaps)
+    finally:
+        close(heaps)
+
+
 def test_put_and_get_move_one_block(lib):
     from tileccl_amd.primitives import copy_block, get, put
 

@@ -142,3 +142,20 @@ def test_standalone_collectives_against_element_loops():
     # (primitives/collectives.py:2536-2545); on values exact in fp16 both orders agree
     plain = halves[0] + halves[1] + halves[2]
     assert torch.equal(ar[0], plain)
+
+
+def test_staged_allreduce_restatement_is_pinned_without_its_own_formula():
+    """Ascending-rank fp32 sum, one rounding: exact integer sums; equal to the reduce-scatter based
+    all-reduce for two ranks (two addends commute); and a three-rank case where rounding after
+    every addition in fp16 (what a dropped fp32 accumulator would do) gives a different answer."""
+    g = torch.Generator().manual_seed(3)
+    ints = [torch.randint(-100, 100, (64,), generator=g).half() for _ in range(4)]
+    assert oc.allreduce_staged(ints)[2].tolist() == [float(sum(int(t[i]) for t in ints)) for i in range(64)]
+    two = [torch.randn(256, generator=g).half() for _ in range(2)]
+    assert torch.equal(oc.allreduce_staged(two)[1], oc.allreduce(two)[0])
+    # 2048 + 1 + 1: fp16 spacing at 2048 is 2, so adding one at a time in fp16 stays at 2048,
+    # while the fp32 sum 2050 is representable
+    three = [torch.tensor([2048.0]).half(), torch.tensor([1.0]).half(), torch.tensor([1.0]).half()]
+    got = oc.allreduce_staged(three)
+    assert all(t.item() == 2050.0 for t in got)
+    assert ((three[0] + three[1]) + three[2]).item() == 2048.0

@@ -144,6 +144,10 @@ SIGNATURES = {
         C.c_int,
         [_vp, _i32, _i64, _vp, _i32, _i64, _i32, _i32, _P(HeapView), _P(TransportDesc), _i32, _vp],
     ),
+    "tccl_allreduce_staged": (
+        C.c_int,
+        [_vp, _i32, _i64, _vp, _vp, _vp, _i32, _i32, _i32, C.c_uint32, _P(HeapView), _vp, _i64, _vp],
+    ),
     "tccl_gemm_allscatter": (
         C.c_int,
         [_P(GemmDesc), _P(ScatterDesc), _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _vp],

@@ -12,6 +12,7 @@
 #include "tccl_comm.h"
 #include "tccl_gemm.h"
 #include "tccl_gemm256.h"
+#include "tccl_staged.h"
 
 namespace {
 
@@ -148,6 +149,22 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
 __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   __shared__ int word[4];
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
+}
+
+// Staged all-reduce: workgroup w carries slot w % slots of the (w / slots)-th rank named in a.ranks.
+__global__ __launch_bounds__(256) void staged_allreduce_kernel(tccl::StagedArgs a) {
+  __shared__ int word;
+  int which = (int)blockIdx.x / a.slots, r = 0;
+  for (; r < a.world; ++r)
+    if (((a.ranks >> r) & 1u) && which-- == 0) break;
+  if (r >= a.world) return;
+  const int slot = (int)blockIdx.x % a.slots;
+  if (a.dtype == tccl::kF16)
+    tccl::staged_role<_Float16>(a, r, slot, &word);
+  else if (a.dtype == tccl::kBF16)
+    tccl::staged_role<__bf16>(a, r, slot, &word);
+  else
+    tccl::staged_role<float>(a, r, slot, &word);
 }
 
 __global__ void fill_kernel(int32_t* w, int64_t n, int32_t v) {
@@ -1138,6 +1155,52 @@ static int allscatter_impl(const tccl_gemm_desc* d, const tccl_scatter_desc* sc,
   c.dst_col_off = sc->dst_col_offset;
   if ((rc = set_task_units(&c, tr, false))) return rc;
   return run_variant(d, c, sync, tr, variant, dev, g, stream, gather, heap);
+}
+
+int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* staging, int32_t* published, int32_t* consumed,
+                          int32_t chunk_elems, int32_t slots, int32_t base_epoch, uint32_t ranks, const tccl_heap_view* heap,
+                          int64_t* fault, int64_t spin_limit_ns, void* stream) {
+  int rc = check_heap(heap);
+  if (rc) return rc;
+  const int esize = (int)dtype_size(dtype);
+  if (dtype != TCCL_F16 && dtype != TCCL_BF16 && dtype != TCCL_F32) return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: dtype %d", dtype);
+  if (!tensor || !staging || !published || !consumed || numel <= 0 || chunk_elems <= 0 || slots <= 0 || base_epoch < 1)
+    return fail(TCCL_ERR_INVALID, "allreduce_staged: bad arguments");
+  const int per_unit = 16 / esize;
+  if (numel % per_unit || chunk_elems % per_unit || !aligned16(tensor) || !aligned16(staging))
+    return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: tensor and chunk must be whole 16-byte units (%d elements)", per_unit);
+  if ((int64_t)chunk_elems * esize > 0x7fffffffll) return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: chunk too large");
+  if (heap->world_size < 32 && (ranks >> heap->world_size)) return fail(TCCL_ERR_INVALID, "allreduce_staged: ranks=0x%x names ranks beyond world_size=%d", ranks, heap->world_size);
+  const int roles = __builtin_popcount(ranks);
+  if (roles == 0) return 0;
+  const int64_t chunks = (numel + chunk_elems - 1) / chunk_elems;
+  if ((int64_t)base_epoch + chunks > 0x7fffffffll) return fail(TCCL_ERR_INVALID, "allreduce_staged: epoch range overflows int32");
+  tccl_device_info dev;
+  if ((rc = query_device(-1, &dev))) return rc;
+  // Every (rank, slot) workgroup waits on others of the same launch: all must be resident.
+  if ((int64_t)roles * slots > (int64_t)dev.compute_units * 4)
+    return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: %d roles x %d slots exceed what the device keeps resident (%d workgroups)", roles,
+                slots, dev.compute_units * 4);
+  tccl::StagedArgs a;
+  memset(&a, 0, sizeof a);
+  a.heap_bases = heap->heap_bases;
+  a.rank = heap->rank;
+  a.world = heap->world_size;
+  a.ranks = ranks;
+  a.tensor = (char*)tensor;
+  a.staging = (char*)staging;
+  a.published = published;
+  a.consumed = consumed;
+  a.units = numel / per_unit;
+  a.chunk_units = chunk_elems / per_unit;
+  a.slots = slots;
+  a.base_epoch = base_epoch;
+  a.dtype = dtype;
+  a.fault = fault;
+  a.spin_ticks = (spin_limit_ns > 0 ? spin_limit_ns : kDefaultSpinNs) / 10 + 1;
+  hipLaunchKernelGGL(staged_allreduce_kernel, dim3(roles * slots), dim3(256), 0, (hipStream_t)stream, a);
+  TCCL_HIP(hipGetLastError());
+  return 0;
 }
 
 int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,

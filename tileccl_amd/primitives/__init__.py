@@ -5,6 +5,7 @@ from tileccl_amd.primitives.collectives import (
     MAX_COLLECTIVE_WORLD_SIZE,
     allgather,
     allreduce,
+    allreduce_staged,
     broadcast,
     reduce_scatter,
     scatter,
@@ -15,6 +16,7 @@ __all__ = [
     "MAX_COLLECTIVE_WORLD_SIZE",
     "allgather",
     "allreduce",
+    "allreduce_staged",
     "broadcast",
     "copy_block",
     "get",

@@ -5,8 +5,10 @@ reduce_scatter`` (``/root/reference/tileccl/primitives/collectives.py:1882-2478`
 same argument order, contracts and messages.  The data movement is the reference's
 direct-write / peer-read form (``tile_allgather`` :613-663, ``tile_scatter`` :671-727,
 ``tile_reduce_scatter`` :730-783, ``tile_broadcast`` :791-836) on this package's bulk copy and
-reduce kernels; its chunked and staged multi-process variants (:840-1592) are scheduling of
-the same movement and have no counterpart here.
+reduce kernels.  Its staged peer-read all-reduce (:840-1044: snapshot a chunk, publish an
+epoch, read the peers' snapshots, acknowledge) is ``allreduce_staged``; the other staged
+variants (:1048-1592) are the same slot protocol around the copies above and have no
+counterpart here.
 
 What differs, on purpose:
 
@@ -217,3 +219,126 @@ def allreduce(tensor: torch.Tensor, heap, op: str = "sum") -> None:
     stage = _staging(heap, block, tensor.dtype)
     _reduce_chunk("allreduce", flat, stage, heap, block)
     copy_block(flat[heap.rank * block : (heap.rank + 1) * block], stage, heap, src_rank=heap.rank, dst_ranks=range(world))
+
+
+# ---------------------------------------------------------------------------------------------
+# The staged peer-read all-reduce (reference :840-1044, launcher :1882-1946).
+#
+# A rank's role waits, inside the kernel, for every peer's role of the same call, so the roles
+# cannot run one call after the other as the collectives above do.  With the ranks emulated as
+# slices of one arena, one launch carries all of them ((rank, slot) -> workgroup); a process
+# that owns a single rank of a real multi-GPU job would pass ``ranks=(heap.rank,)``.
+
+STAGED_MIN_CHUNK_BYTES = 16 << 10      # a workgroup's chunk: 4 x 16 bytes per thread ...
+STAGED_MAX_CHUNK_BYTES = 64 << 10      # ... to 16 x 16 bytes
+STAGED_RESIDENT_WORKGROUPS = 1024      # world x slots must be resident at once (4 workgroups on each of 256 CUs)
+STAGED_MAX_PIPELINE_SLOTS = 256        # workgroups per rank
+_DEFAULT_SPIN_NS = 0                   # the library's default bound on a wait
+
+
+class _StagedWorkspace:
+    """Staging rows and the two words per slot, at one offset in every rank's slice, plus the
+    epoch counter of the calls that used them (reference ``_AllReduceWorkspace``, :2813-2838)."""
+
+    def __init__(self, heaps, dtype: torch.dtype, chunk_elems: int, slots: int) -> None:
+        self.staging = [h.allocate_tensor((slots, chunk_elems), dtype) for h in heaps]
+        self.published = [h.allocate_tensor((slots,), torch.int32) for h in heaps]
+        self.consumed = [h.allocate_tensor((slots,), torch.int32) for h in heaps]
+        for group in (self.staging, self.published, self.consumed):
+            offsets = {h.get_offset(int(t.data_ptr())) for h, t in zip(heaps, group)}
+            if len(offsets) != 1:
+                raise RuntimeError("allreduce_staged: the ranks' heaps have diverged, no common workspace offset")
+        for t in self.published + self.consumed:
+            t.zero_()
+        self.fault = torch.zeros(1, dtype=torch.int64, device=self.staging[0].device)
+        self.next_epoch = 1
+
+    def reserve_epoch_range(self, chunks: int) -> int:
+        if self.next_epoch + chunks >= 2**31 - 1:  # start over: no role is in flight between calls on one stream
+            for t in self.published + self.consumed:
+                t.zero_()
+            self.next_epoch = 1
+        base, self.next_epoch = self.next_epoch, self.next_epoch + chunks
+        return base
+
+
+_STAGED: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()  # heap of rank 0 -> {(dtype, chunk, slots): workspace}
+
+
+def resolve_staged_execution(numel: int, element_size: int, world: int, *, chunk_elems: int | None = None,
+                             pipeline_slots: int | None = None) -> tuple[int, int, int]:
+    """(chunk_elems, chunks, pipeline_slots) for a tensor: as many slots as stay resident, at
+    most 256 per rank, and the smallest chunk of 16 / 32 / 64 KiB that gives every slot work
+    (measured on two and four ranks, 1 MiB to 256 MiB: more slots always won; 16 KiB chunks
+    are quickest while the slots outnumber them, 64 KiB chunks from there on).  The reference's
+    policy (:2586-2597) picks 256..4096 elements and at most 16 programs for its target; the
+    contract is the same."""
+    per_unit = 16 // element_size
+    slot_cap = max(1, min(STAGED_MAX_PIPELINE_SLOTS, STAGED_RESIDENT_WORKGROUPS // world))
+    if chunk_elems is None:
+        chunk_bytes = STAGED_MIN_CHUNK_BYTES
+        while chunk_bytes < STAGED_MAX_CHUNK_BYTES and numel * element_size > chunk_bytes * slot_cap:
+            chunk_bytes *= 2
+        chunk_elems = min(chunk_bytes // element_size, -(-numel // per_unit) * per_unit)
+    if chunk_elems <= 0 or chunk_elems % per_unit:
+        raise ValueError(f"allreduce_staged: chunk_elems={chunk_elems} must be a positive multiple of {per_unit}")
+    chunks = -(-numel // chunk_elems)
+    if pipeline_slots is None:
+        pipeline_slots = min(chunks, slot_cap)
+    if pipeline_slots < 1:
+        raise ValueError(f"allreduce_staged: pipeline_slots={pipeline_slots} must be at least 1")
+    return chunk_elems, chunks, min(pipeline_slots, chunks)
+
+
+def allreduce_staged(tensors, heaps, op: str = "sum", *, chunk_elems: int | None = None, pipeline_slots: int | None = None,
+                     ranks=None, spin_limit_ns: int = _DEFAULT_SPIN_NS) -> torch.Tensor:
+    """In place on every rank's tensor, in one launch: each ends with the sum over ranks.
+
+    ``tensors[r]`` is rank ``r``'s tensor in ``heaps[r]``, all at one heap offset.  ``ranks``
+    names the roles the launch carries (default: all).  Returns the fault word of the
+    workspace (int64[1] on the device): non-zero after a wait ran into ``spin_limit_ns``,
+    which is what happens when a role that the others wait for is left out.
+    """
+    if op != "sum":
+        raise ValueError(f"Only op='sum' is currently supported, got {op!r}")
+    world = len(heaps)
+    if len(tensors) != world or any(h.world_size != world or h.rank != r for r, h in enumerate(heaps)):
+        raise ValueError("allreduce_staged expects one tensor and one heap per rank, in rank order")
+    _validate_world_size(world)
+    first = tensors[0]
+    for r, (t, h) in enumerate(zip(tensors, heaps)):
+        _contiguous("allreduce_staged", t, f"tensors[{r}]")
+        _on_heap(t, h, f"tensors[{r}]")
+        if t.dtype != first.dtype or t.shape != first.shape:
+            raise ValueError("allreduce_staged expects one dtype and shape on every rank")
+    if len({h.get_offset(int(t.data_ptr())) for t, h in zip(tensors, heaps)}) != 1:
+        raise ValueError("allreduce_staged expects the tensor at the same heap offset on every rank")
+    if first.dtype not in _REDUCE_IN:
+        raise ValueError(f"allreduce_staged supports fp16, bf16 and fp32 tensors, got {first.dtype}")
+    numel = int(first.numel())
+    carried = tuple(range(world)) if ranks is None else tuple(int(r) for r in ranks)
+    for r in carried:
+        _validate_root(r, world_size=world)
+    cache = _STAGED.setdefault(heaps[0], {})
+    if world == 1 or numel == 0 or not carried:
+        return torch.zeros(1, dtype=torch.int64, device=first.device)  # local identity (reference :2563-2583)
+    _whole_units("allreduce_staged", numel, first.element_size())
+    chunk_elems, chunks, slots = resolve_staged_execution(numel, first.element_size(), world, chunk_elems=chunk_elems,
+                                                          pipeline_slots=pipeline_slots)
+    key = (str(first.dtype), chunk_elems, slots)
+    if key not in cache:
+        cache[key] = _StagedWorkspace(heaps, first.dtype, chunk_elems, slots)
+    ws = cache[key]
+    base_epoch = ws.reserve_epoch_range(chunks)
+    ws.fault.zero_()
+    view = _launch.heap_view(heaps[0].get_heap_bases(), 0, world)
+    mask = 0
+    for r in carried:
+        mask |= 1 << r
+    rc = _lib.load().tccl_allreduce_staged(
+        _launch.ptr(tensors[0]), _launch.dtype_code(first.dtype), numel, _launch.ptr(ws.staging[0]), _launch.ptr(ws.published[0]),
+        _launch.ptr(ws.consumed[0]), chunk_elems, slots, base_epoch, mask, _launch.byref(view), _launch.ptr(ws.fault),
+        int(spin_limit_ns), _launch.stream_ptr(),
+    )
+    _lib.check(rc, "tccl_allreduce_staged")
+    return ws.fault
