@@ -128,12 +128,13 @@ def launch_spread(run, variant, launches=100):
 class Workload:
     """One benchmark configuration: heap slices, resident inputs, the fused operation."""
 
-    def __init__(self, name, macro_tile, group_tiles=None):
+    def __init__(self, name, macro_tile, group_tiles=None, b_layout="kn"):
         import torch
 
         from tileccl_amd.v2 import FusedGemmAllGather, FusedGemmReduceScatter, SymmetricHeap
 
         self.name = name
+        self.b_layout = b_layout
         self.kind, self.M, self.N, self.K, self.block_m, self.in_type = WORKLOADS[name]
         M, N, K = self.M, self.N, self.K
         self.group_tiles, self.calibration = self.resolve_group_tiles(group_tiles)
@@ -174,7 +175,10 @@ class Workload:
             self.exchange_bytes = 2.0 * M * N * psz + M * N * 2  # both partials read once, every output row written once
         self.op = self.ops[0]
         self.A = self.heaps[0].allocate_tensor((M, K), self.A_cpu.dtype)
-        self.B = self.heaps[0].allocate_tensor((K, N), self.B_cpu.dtype)
+        if b_layout == "nk":  # the same B held as an (N, K) tensor, handed over as its `.t()` view
+            self.B = self.heaps[0].allocate_tensor((N, K), self.B_cpu.dtype).t()
+        else:
+            self.B = self.heaps[0].allocate_tensor((K, N), self.B_cpu.dtype)
         self.A.copy_(self.A_cpu)
         self.B.copy_(self.B_cpu)
         self.op.mark_peers_ready()
@@ -407,6 +411,9 @@ def main() -> int:
     ap.add_argument("--group-tiles", default="default",
                     help="tiles per TileGroup: 'default' (the planner's rule), 'auto' (calibrate this machine and ask the "
                          "cost model), or a number")
+    ap.add_argument("--b-layout", default="kn", choices=["kn", "nk"],
+                    help="B in memory: 'kn' = (K, N) row-major (the configurations' layout), 'nk' = an (N, K) tensor passed "
+                         "as its .t() view (a linear layer's weight)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -422,7 +429,7 @@ def main() -> int:
     if WORKLOADS[args.workload][0] == "ch":
         w = ChainedWorkload(args.workload, args.macro_tile)
     else:
-        w = Workload(args.workload, args.macro_tile, args.group_tiles)
+        w = Workload(args.workload, args.macro_tile, args.group_tiles, args.b_layout)
 
     results = {}
     wanted = [v for v in ("s0", "s1", "s2") if v in args.variants.split(",") or v == args.variant]
@@ -482,12 +489,14 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.variant, args.macro_tile))
-            if args.group_tiles == "default" else None,
+            if args.group_tiles == "default" and args.b_layout == "kn" else None,
             "kernel_ms": round(chosen["event_ms_mean"], 5),
         },
     }
     if getattr(w, "calibration", None):
         line["config"]["calibration"] = w.calibration
+    if args.b_layout != "kn":
+        line["config"]["b_layout"] = "B held as (N, K), passed as its .t() view"
     if push_only is not None:
         line["one_direction"] = push_only
     if "s0" in results and "s2" in results:

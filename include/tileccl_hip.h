@@ -104,6 +104,11 @@ typedef struct tccl_gemm_desc {
  * (The reference's fused proof kernels have no counterpart in its tree; tile_reduce_scatter,
  * primitives/collectives.py:730-783, always reads a stored partial.) */
 #define TCCL_GEMM_OWN_ROWS_IN_REGISTERS 1
+/* B is k-major: element (k, n) is at B[n * ldb + k], i.e. B is the `.t()` view of an (N, K)
+ * tensor (the layout of a linear layer's weight); ldb is then the pitch between columns and must
+ * be >= K.  The reference's GEMM takes arbitrary strides (kernels/gemm.py:139-151); this and the
+ * row-major form are the two it meets in practice.  With column_shards = w, B has w * N columns. */
+#define TCCL_GEMM_B_KMAJOR 2
 
 #define TCCL_RS_EMULATE_PEERS 1
 #define TCCL_RS_PEERS_RESIDENT 2

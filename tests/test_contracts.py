@@ -218,3 +218,24 @@ def test_staged_allreduce_execution_policy():
         resolve(4096, 2, 2, chunk_elems=100)
     with pytest.raises(ValueError, match="at least 1"):
         resolve(4096, 2, 2, pipeline_slots=0)
+
+
+def test_b_operand_layouts():
+    """Row-major B, or the transposed view of a row-major tensor (k-major); anything else is refused."""
+    import pytest
+    import torch
+
+    from tileccl_amd import _launch, _lib
+
+    B = torch.zeros(64, 128, dtype=torch.float16)
+    assert _launch._b_layout(B) == (128, 0)
+    assert _launch._b_layout(torch.zeros(64, 256, dtype=torch.float16)[:, :128]) == (256, 0)
+    W = torch.zeros(128, 64, dtype=torch.float16)  # (N, K)
+    assert _launch._b_layout(W.t()) == (64, _lib.GEMM_B_KMAJOR)
+    assert _launch._b_layout(torch.zeros(128, 72, dtype=torch.float16)[:, :64].t()) == (72, _lib.GEMM_B_KMAJOR)
+    assert _launch._b_layout(torch.zeros(64, 1, dtype=torch.float16)) == (1, 0)  # one column: row-major
+    assert _launch._b_layout(torch.zeros(8, 1, dtype=torch.float16).t()) == (8, 0)  # (1, 8): one row, contiguous
+    with pytest.raises(ValueError, match="contiguous rows or be the transposed view"):
+        _launch._b_layout(torch.zeros(64, 256, dtype=torch.float16)[:, ::2])
+    with pytest.raises(ValueError, match="2-D"):
+        _launch._b_layout(torch.zeros(4, 4, 4))

@@ -14,10 +14,18 @@ from tests.gpu_util import assert_gemm_close, seeded
 pytestmark = pytest.mark.gpu
 
 
-def run_gemm(lib, A_cpu, B_cpu, out_dtype, **kw):
+def k_major(B_cpu, pad=0):
+    """B on the device as the transposed view of an (N, K + pad) tensor: element (k, n) at n * (K + pad) + k."""
+    K, N = B_cpu.shape
+    backing = torch.zeros(N, K + pad, dtype=B_cpu.dtype, device="cuda")
+    backing[:, :K] = B_cpu.t().cuda()
+    return backing[:, :K].t()
+
+
+def run_gemm(lib, A_cpu, B_cpu, out_dtype, b_kmajor=False, b_pad=0, **kw):
     from tileccl_amd import _launch, _lib
 
-    A, B = A_cpu.cuda(), B_cpu.cuda()
+    A, B = A_cpu.cuda(), (k_major(B_cpu, b_pad) if b_kmajor else B_cpu.cuda())
     out = torch.full((A.shape[0], B.shape[1]), float("nan"), dtype=out_dtype, device="cuda")
     desc = _launch.gemm_desc(A, B, out, **kw)
     _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
@@ -56,6 +64,24 @@ def test_gemm_matches_fp32_matmul(lib, M, N, K, dtype, macro):
     # which can flip a rounding, so allow one output ulp against it
     want = oracle.gemm(A, B, dtype)
     assert (got.cpu().float() - want.float()).abs().max().item() <= (0.004 if dtype == torch.float16 else 0.032)
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES + [(512, 520, 1000)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("macro", MACRO)
+def test_k_major_B_gives_the_bits_of_row_major_B(lib, M, N, K, dtype, macro):
+    """B handed over as the `.t()` view of an (N, K) tensor (a linear layer's weight): the k order of
+    the sums does not depend on the layout, so the result is bit-identical to the row-major run;
+    with a padded pitch too (ldb = K + 8)."""
+    A = seeded((M, K), 0, dtype)
+    B = seeded((K, N), 1, dtype, scale=K**-0.5)
+    want = run_gemm(lib, A, B, dtype, macro_tile=macro)
+    assert_gemm_close(want, A.float() @ B.float(), tight=0.004 if dtype == torch.float16 else 0.032)
+    for pad in (0, 8):
+        got = run_gemm(lib, A, B, dtype, b_kmajor=True, b_pad=pad, macro_tile=macro)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), pad
+    got32 = run_gemm(lib, A, B, torch.float32, b_kmajor=True, macro_tile=macro)
+    assert torch.equal(got32, run_gemm(lib, A, B, torch.float32, macro_tile=macro))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -108,7 +134,14 @@ def test_unsupported_layouts_fail_loudly(lib):
     A, B = seeded((128, 64), 0).cuda(), seeded((64, 128), 1).cuda()
     out = torch.empty(128, 128, dtype=torch.float16, device="cuda")
     with pytest.raises(ValueError, match="contiguous rows"):
-        _launch.gemm_desc(A, B.t().contiguous().t(), out)
+        _launch.gemm_desc(A, torch.empty(64, 256, dtype=torch.float16, device="cuda")[:, ::2], out)
+    with pytest.raises(ValueError, match="contiguous rows"):
+        _launch.gemm_desc(A.t().contiguous().t(), B, out)
+    with pytest.raises(ValueError, match="leading dimension smaller"):
+        d = _launch.gemm_desc(A, B, out)
+        d.flags |= _lib.GEMM_B_KMAJOR  # row-major pitch (128) read as a k-major one is fine; K = 64 <= 128
+        d.ldb = 32
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
     with pytest.raises(ValueError, match="K=60 must be a multiple of 8"):
         d = _launch.gemm_desc(A[:, :60].contiguous(), B[:60].contiguous(), out)
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")

@@ -53,6 +53,24 @@ def _row_major(t: torch.Tensor, name: str) -> int:
     return int(t.stride(0)) if t.shape[0] > 1 else int(t.shape[1])
 
 
+def _b_layout(B: torch.Tensor) -> tuple[int, int]:
+    """(ldb, flag bits) of the B operand: rows contiguous, or the ``.t()`` view of a tensor whose
+    rows are contiguous (k-major: the layout of a linear layer's weight).  The reference's kernels
+    take any strides (``/root/reference/tileccl/kernels/gemm.py:139-151``); these are the two forms
+    with 16-byte vector access."""
+    if B.ndim != 2:
+        raise ValueError(f"B must be 2-D, got {B.ndim}-D")
+    K, N = B.shape
+    if N == 1 or B.stride(1) == 1:
+        return _row_major(B, "B"), 0
+    if K == 1 or B.stride(0) == 1:
+        return (int(B.stride(1)) if N > 1 else int(K)), _lib.GEMM_B_KMAJOR
+    raise ValueError(
+        f"B must have contiguous rows or be the transposed view of such a tensor, got strides {tuple(B.stride())}; "
+        "call .contiguous() first"
+    )
+
+
 def gemm_desc(
     A: torch.Tensor,
     B: torch.Tensor,
@@ -84,13 +102,14 @@ def gemm_desc(
     d = _lib.GemmDesc()
     d.A, d.B, d.C = ptr(A), ptr(B), ptr(C_out)
     d.M, d.N, d.K = int(M), int(N), int(K)
-    d.lda, d.ldb, d.ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C_out, "C")
+    ldb, b_flags = _b_layout(B)
+    d.lda, d.ldb, d.ldc = _row_major(A, "A"), ldb, _row_major(C_out, "C")
     d.in_dtype, d.out_dtype = dtype_code(A.dtype), dtype_code(C_out.dtype)
     d.alpha = float(alpha)
     d.block_m, d.block_n, d.group_m = int(block_m), int(block_n), int(group_m)
     d.num_wgs = int(num_wgs)
     d.macro_tile = int(macro_tile)
-    d.flags = int(flags)
+    d.flags = int(flags) | b_flags
     d.column_shards = int(column_shards)
     return d
 

@@ -62,6 +62,7 @@ class GemmDesc(C.Structure):
 
 
 GEMM_OWN_ROWS_IN_REGISTERS = 1  # TCCL_GEMM_OWN_ROWS_IN_REGISTERS
+GEMM_B_KMAJOR = 2  # TCCL_GEMM_B_KMAJOR
 
 
 class SyncDesc(C.Structure):

@@ -2,27 +2,30 @@
 
     python -m tileccl_amd.csrc.build
 
-The library is a single translation unit (``tccl_api.hip`` plus headers).  It is built
-next to the Python package so that it travels with the source tree.
+The library is two translation units (``tccl_api.hip``: entry points and the kernels for
+row-major B; ``tccl_kmajor.hip``: the large-tile kernels for k-major B) compiled side by side
+and linked.  It is built next to the Python package so that it travels with the source tree.
 """
 
 from __future__ import annotations
 
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 HERE = Path(__file__).resolve().parent
 OUT = HERE.parent / "libtileccl_hip.so"
-SOURCES = [HERE / "tccl_api.hip"]
-HEADERS = [HERE / "tccl_device.h", HERE / "tccl_gemm.h", HERE / "tccl_gemm256.h", HERE / "tccl_comm.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
+SOURCES = [HERE / "tccl_api.hip", HERE / "tccl_kmajor.hip"]
+HEADERS = [HERE / "tccl_device.h", HERE / "tccl_gemm.h", HERE / "tccl_gemm256.h", HERE / "tccl_kernels256.h", HERE / "tccl_comm.h",
+           HERE / "tccl_staged.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
 
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-Wno-comment",
     # hipcc -O3 must not form packed-fp32 instructions on this hardware pool.
     "-Xclang",
@@ -32,9 +35,7 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = False, extra: list[str] | None = None) -> Path:
-    """Compile unconditionally; raises ``RuntimeError`` with the compiler output on failure."""
-    cmd = ["hipcc", *FLAGS, *(extra or []), *map(str, SOURCES), "-o", str(OUT)]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, cwd=HERE, capture_output=True, text=True)
@@ -43,6 +44,20 @@ def build(verbose: bool = False, extra: list[str] | None = None) -> Path:
     if verbose and proc.stderr:
         # The host pass reports the packed-fp32 feature as unknown; that is expected.
         print(proc.stderr, file=sys.stderr)
+
+
+def build(verbose: bool = False, extra: list[str] | None = None) -> Path:
+    """Compile unconditionally; raises ``RuntimeError`` with the compiler output on failure."""
+    with tempfile.TemporaryDirectory(prefix="tccl_build_") as tmp:
+        objects = [str(Path(tmp) / (src.stem + ".o")) for src in SOURCES]
+        with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
+            jobs = [
+                pool.submit(_run, ["hipcc", *FLAGS, *(extra or []), "-c", str(src), "-o", obj], verbose)
+                for src, obj in zip(SOURCES, objects)
+            ]
+            for job in jobs:
+                job.result()
+        _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", str(OUT)], verbose)
     return OUT
 
 

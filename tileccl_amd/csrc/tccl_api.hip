@@ -12,9 +12,12 @@
 #include "tccl_comm.h"
 #include "tccl_gemm.h"
 #include "tccl_gemm256.h"
+#include "tccl_kernels256.h"
 #include "tccl_staged.h"
 
 namespace {
+
+using tccl::Fused256Args;
 
 thread_local char g_error[512] = "";
 
@@ -96,56 +99,6 @@ __global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::S
   }
 }
 
-// Large-tile GEMM: 512 threads, one workgroup per CU, both LDS stages resident.
-template <typename InT, typename OutT>
-__global__ __launch_bounds__(512, 2) void gemm256_kernel(tccl::GemmArgs g, tccl::Macro m) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
-  __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
-  tccl::warm_kernargs<(int)(sizeof(tccl::GemmArgs) + sizeof(tccl::Macro))>();
-  tccl::SignalArgs s;
-  s.mode = tccl::kSignalNone;
-  tccl::Gemm256<InT, OutT>(g, -1, -1, -1, stage0, stage1, nullptr).run(s, m, (int)blockIdx.x, (int)gridDim.x);
-#endif
-}
-
-// Large-tile GEMM whose workgroups, once their tiles are stored (and pushed to the peers
-// from the epilogue), turn into the communication role.  The tile fills a CU's LDS and
-// registers, so no separate communication workgroup could share the CU with it; instead
-// every workgroup produces first and moves data afterwards.  No workgroup waits before its
-// own tiles are published and the grid never exceeds the CU count, so every wait is on a
-// workgroup that is running.  `push` and `comm` are read from the argument block at their
-// point of use (late_kernarg), never through the parameter itself.
-struct Fused256Args {
-  tccl::GemmArgs g;
-  tccl::SignalArgs s;
-  tccl::Macro m;
-  int64_t* trace_start;
-  tccl::PullArgs pull;
-  tccl::PushArgs push;
-  tccl::ReduceArgs reduce;
-  tccl::GatherArgs gather;
-  tccl::CommArgs comm;
-};
-
-template <typename InT, typename OutT, bool kWithReduce, bool kGatherA = false>
-__global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __shared__ __attribute__((aligned(16))) char stage0[tccl::kStage256];
-  __shared__ __attribute__((aligned(16))) char stage1[tccl::kStage256];
-  __shared__ __attribute__((aligned(16))) char landing_words[tccl::kBgWordBytes];
-  tccl::warm_kernargs<(int)sizeof(Fused256Args)>();
-  if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = tccl::now_ticks();
-  tccl::Gemm256<InT, OutT, kWithReduce, kGatherA>(f.g, (int)offsetof(Fused256Args, pull), (int)offsetof(Fused256Args, push),
-                                                  (int)offsetof(Fused256Args, reduce), stage0, stage1, landing_words,
-                                                  (int)offsetof(Fused256Args, gather))
-      .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
-  __syncthreads();
-  const tccl::CommArgs c = tccl::late_kernarg<tccl::CommArgs>((int)offsetof(Fused256Args, comm));
-  tccl::comm_role<tccl::kThreads256>(c, (int)blockIdx.x, (int)gridDim.x, (int*)stage1);
-#endif
-}
-
 __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   __shared__ int word[4];
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
@@ -212,13 +165,15 @@ int check_gemm(const tccl_gemm_desc* d) {
   const int in_vec = (int)(16 / isz), out_vec = (int)(16 / osz);
   if (d->K % in_vec) return fail(TCCL_ERR_UNSUPPORTED, "gemm: K=%d must be a multiple of %d", d->K, in_vec);
   if (d->N % 8) return fail(TCCL_ERR_UNSUPPORTED, "gemm: N=%d must be a multiple of 8", d->N);
-  if (d->lda < d->K || d->ldb < (int64_t)d->N * shards || d->ldc < d->N) return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
+  const bool b_kmajor = (d->flags & TCCL_GEMM_B_KMAJOR) != 0;
+  if (d->lda < d->K || d->ldb < (b_kmajor ? (int64_t)d->K : (int64_t)d->N * shards) || d->ldc < d->N)
+    return fail(TCCL_ERR_INVALID, "gemm: leading dimension smaller than the row length");
   if (d->lda % in_vec || d->ldb % in_vec || d->ldc % out_vec || !aligned16(d->A) || !aligned16(d->B) || !aligned16(d->C))
     return fail(TCCL_ERR_UNSUPPORTED, "gemm: A, B, C rows must start on 16-byte boundaries");
   // The kernels address an operand with 32-bit byte offsets from a per-tile base: B from its
-  // first row down to row K-1, A and C over the 256 rows of a tile.
+  // first row down to row K-1 (k-major B: over the 256 columns of a tile), A and C over the 256 rows of a tile.
   const int64_t limit = 0xffffffffll;
-  const int64_t b_span = ((int64_t)(d->K - 1) * d->ldb + (int64_t)d->N * shards) * (int64_t)isz;
+  const int64_t b_span = (b_kmajor ? 255 * d->ldb + d->K : (int64_t)(d->K - 1) * d->ldb + (int64_t)d->N * shards) * (int64_t)isz;
   const int64_t a_span = (255 * d->lda + d->K) * (int64_t)isz;
   const int64_t c_span = (255 * d->ldc + d->N) * (int64_t)osz;
   if (b_span > limit || a_span > limit || c_span > limit)
@@ -256,6 +211,7 @@ int build_gemm_args(const tccl_gemm_desc* d, const tccl_device_info& dev, tccl::
   g->xcds = dev.xcds;
   g->span = gemm_span(d->group_m * g->tile_cols, d->group_m, g->tile_cols, dev.xcds);
   g->wrap_rows = d->column_shards > 1 ? d->M / d->column_shards : 0;
+  g->b_kmajor = (d->flags & TCCL_GEMM_B_KMAJOR) ? 1 : 0;
   return 0;
 }
 
@@ -394,51 +350,24 @@ int default_macro_wgs(const tccl_gemm_desc* d, const tccl_device_info& dev) {
   return n < 1 ? 1 : n;
 }
 
-template <typename InT, typename OutT>
-int launch_gemm256_t(const tccl::GemmArgs& g, const tccl::Macro& m, int wgs, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm256_kernel<InT, OutT>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, g, m);
-  TCCL_HIP(hipGetLastError());
-  return 0;
+// Large-tile kernels: B row-major ones are instantiated here, the k-major ones in tccl_kmajor.hip.
+int launch_status(int rc, int in_dtype, int out_dtype) {
+  if (rc == 0) return 0;
+  if (rc == tccl::kNoKernel) return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
+  if (rc == tccl::kGatherTypes) return fail(TCCL_ERR_UNSUPPORTED, "gathered input read in place: output type must equal the input type, B row-major");
+  return hip_fail((hipError_t)rc, "large-tile kernel launch");
 }
 
 int launch_gemm256(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tccl::Macro& m, int wgs, hipStream_t stream) {
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_gemm256_t<_Float16, _Float16>(g, m, wgs, stream);
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_gemm256_t<_Float16, float>(g, m, wgs, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_gemm256_t<__bf16, __bf16>(g, m, wgs, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_gemm256_t<__bf16, float>(g, m, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_BF16) return launch_gemm256_t<tccl::fp8e4m3, __bf16>(g, m, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F16) return launch_gemm256_t<tccl::fp8e4m3, _Float16>(g, m, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F32) return launch_gemm256_t<tccl::fp8e4m3, float>(g, m, wgs, stream);
-  return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
-}
-
-template <typename InT, typename OutT>
-int launch_fused256_t(const Fused256Args& f, int wgs, hipStream_t stream) {
-  // The tile-by-tile reduce-scatter is a separate instantiation: its code would otherwise
-  // raise the register pressure of every fused kernel.
-  if (f.gather.active) {
-    // Instantiated for outputs of the input type only (gather_in_place() admits nothing else).
-    if constexpr (std::is_same<InT, OutT>::value)
-      hipLaunchKernelGGL((fused256_kernel<InT, OutT, false, true>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
-    else
-      return fail(TCCL_ERR_UNSUPPORTED, "gathered input read in place: output type must equal the input type");
-  } else if (f.reduce.active)
-    hipLaunchKernelGGL((fused256_kernel<InT, OutT, true>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
-  else
-    hipLaunchKernelGGL((fused256_kernel<InT, OutT, false>), dim3(wgs), dim3(tccl::kThreads256), 0, stream, f);
-  TCCL_HIP(hipGetLastError());
-  return 0;
+  const int rc = g.b_kmajor ? tccl::launch_gemm256_kmajor(in_dtype, out_dtype, g, m, wgs, stream)
+                            : tccl::launch_gemm256_table<false>(in_dtype, out_dtype, g, m, wgs, stream);
+  return launch_status(rc, in_dtype, out_dtype);
 }
 
 int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs, hipStream_t stream) {
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_fused256_t<_Float16, _Float16>(f, wgs, stream);
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused256_t<_Float16, float>(f, wgs, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused256_t<__bf16, __bf16>(f, wgs, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused256_t<__bf16, float>(f, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_BF16) return launch_fused256_t<tccl::fp8e4m3, __bf16>(f, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F16) return launch_fused256_t<tccl::fp8e4m3, _Float16>(f, wgs, stream);
-  if (in_dtype == TCCL_F8E4M3 && out_dtype == TCCL_F32) return launch_fused256_t<tccl::fp8e4m3, float>(f, wgs, stream);
-  return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
+  const int rc = f.g.b_kmajor ? tccl::launch_fused256_kmajor(in_dtype, out_dtype, f, wgs, stream)
+                              : tccl::launch_fused256_table<false>(in_dtype, out_dtype, f, wgs, stream);
+  return launch_status(rc, in_dtype, out_dtype);
 }
 
 // The pull half of a TileGroup all-gather, as the large-tile K loop performs it in the
@@ -623,7 +552,7 @@ void build_gather_background(const tccl_gemm_desc* d, const GatherSpec& gs, cons
 bool gather_in_place(const tccl_gemm_desc* d, const tccl_device_info& dev, int k_shard, int variant) {
   if (variant == TCCL_S0_BULK || !use_macro(d, dev)) return false;
   if (d->in_dtype != d->out_dtype || (d->in_dtype != TCCL_F16 && d->in_dtype != TCCL_BF16)) return false;
-  return k_shard % 64 == 0 && d->column_shards <= 1;
+  return k_shard % 64 == 0 && d->column_shards <= 1 && !(d->flags & TCCL_GEMM_B_KMAJOR);
 }
 
 // GEMM (+ optional communication role) for one of the three operations.

@@ -12,6 +12,8 @@
 //   A (M x K, k-contiguous) lands in that layout directly.  B (K x N, n-contiguous) is
 //   transposed in registers on the way in: a thread owns a 4(k) x 8(n) patch, repacks it
 //   to 8 x (4 consecutive k) and writes eight 8-byte words.
+//   A k-major B (GemmArgs::b_kmajor: element (k, n) at B[n * ldb + k]) takes A's route: loaded
+//   by rows of n, it is already in the k-chunked layout.
 //   LDS is single-buffered; the next K step's global loads are issued before the MFMAs
 //   of the current one, so two workgroups per CU keep the matrix cores fed.
 //
@@ -57,6 +59,8 @@ struct GemmArgs {
   // Column shards stacked as row blocks (0: plain GEMM): C row block q of wrap_rows rows is
   // A (wrap_rows x K) times columns [q * N, (q + 1) * N) of B; tiles never straddle two blocks.
   int wrap_rows;
+  // B is k-major: element (k, n) at B[n * ldb + k] (the `.t()` view of an (N, K) tensor).
+  int b_kmajor;
 };
 
 // Where a tile whose first output row is row0 and first output column col0 reads its operands.
@@ -153,16 +157,18 @@ struct GemmRole {
     Source s;
     const OperandOrigin o = operand_origin(g, row0, col0);
     const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
-    const InT* B = (const InT*)g.B + o.b_col;
+    const InT* B = (const InT*)g.B + (g.b_kmajor ? (int64_t)o.b_col * g.ldb : (int64_t)o.b_col);
     s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * kEsz), 0x00020000);
-    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
+    const int64_t b_elems = g.b_kmajor ? (int64_t)(o.b_cols - 1 - o.b_col) * g.ldb + g.K : (int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col);
+    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(b_elems * kEsz), 0x00020000);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       s.off_a[i] = (uint32_t)(((tid >> 3) + 32 * i) * g.lda * kEsz + (tid & 7) * 16);
-      s.off_b[i] = (uint32_t)(((tid >> 4) * 4 + i) * g.ldb * kEsz + (tid & 15) * 16);
+      s.off_b[i] = g.b_kmajor ? (uint32_t)(((tid >> 3) + 32 * i) * g.ldb * kEsz + (tid & 7) * 16)
+                              : (uint32_t)(((tid >> 4) * 4 + i) * g.ldb * kEsz + (tid & 15) * 16);
     }
     s.step_a = kBK * kEsz;
-    s.step_b = (uint32_t)(kBK * g.ldb * kEsz);
+    s.step_b = g.b_kmajor ? (uint32_t)(kBK * kEsz) : (uint32_t)(kBK * g.ldb * kEsz);
     return s;
   }
 
@@ -176,8 +182,9 @@ struct GemmRole {
       const uint32_t off = dead ? 0xfffffff0u : s.off_a[i] + adv_a;
       ra[i] = __builtin_amdgcn_raw_buffer_load_b128(s.a, off, 0, 0);
     }
+    const bool dead_b = dead && g.b_kmajor;  // row-major B: rows >= K lie past the end of the buffer
 #pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(s.b, s.off_b[i] + adv_b, 0, 0);
+    for (int i = 0; i < 4; ++i) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(s.b, dead_b ? 0xfffffff0u : s.off_b[i] + adv_b, 0, 0);
   }
 
   // ---- registers -> LDS ---------------------------------------------------------------
@@ -186,6 +193,12 @@ struct GemmRole {
 #pragma unroll
     for (int i = 0; i < 4; ++i) *(u32x4*)(la + ((tid >> 3) + 32 * i) * 16) = ra[i];
 
+    if (g.b_kmajor) {  // rb[i]: the 8 consecutive k of column (tid >> 3) + 32 * i, as the reads want them
+      char* lb = lds + kOperandBytes + (tid & 7) * kPlane;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *(u32x4*)(lb + b_slot((tid >> 3) + 32 * i) * 16) = rb[i];
+      return;
+    }
     // rb[i] holds columns n0..n0+7 of k row i as 4 dwords (two columns each).  Column
     // n0+j needs its four k values side by side: two dwords (k0|k1) and (k2|k3).
     const int kg = tid >> 4;

@@ -227,7 +227,11 @@ TCCL_D void warm_kernargs() {
   asm volatile("" ::"s"(any));
 }
 
-template <typename InT, typename OutT, bool kWithReduce = false, bool kGatherA = false>
+// kBKMajor: B is given with k contiguous (element (k, n) at B[n * ldb + k], what a `.t()` view of
+// an (N, K) weight is: the reference's kernels take any strides, kernels/gemm.py:139-151).  The B
+// stage then has the A stage's layout (256 n rows of 128 bytes, same swizzle) and is read with
+// ds_read_b128 like A: no transposing reads.
+template <typename InT, typename OutT, bool kWithReduce = false, bool kGatherA = false, bool kBKMajor = false>
 struct Gemm256 {
   typedef typename Mfma<InT>::Vec Vec;
   static constexpr int kEszIn = sizeof(InT);
@@ -311,9 +315,12 @@ struct Gemm256 {
     Source s;
     const OperandOrigin o = operand_origin(g, row0, col0);
     const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
-    const InT* B = (const InT*)g.B + o.b_col;
+    const InT* B = (const InT*)g.B + (kBKMajor ? (int64_t)o.b_col * g.ldb : (int64_t)o.b_col);
     s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * kEsz), 0x00020000);
-    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
+    if constexpr (kBKMajor)
+      s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(o.b_cols - 1 - o.b_col) * g.ldb + g.K) * kEsz), 0x00020000);
+    else
+      s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = 8 * (4 * wave + i) + (lane >> 3);
@@ -321,7 +328,9 @@ struct Gemm256 {
       int64_t lda = g.lda;
       if constexpr (kGatherA) lda = late_kernarg_ptr<GatherArgs>(gather_offset)->ld_shard;
       s.off_a[i] = (uint32_t)(row * lda * kEsz + kc * 16);
-      if constexpr (kFp8) {
+      if constexpr (kBKMajor) {
+        s.off_b[i] = (uint32_t)(row * g.ldb * kEsz + kc * 16);
+      } else if constexpr (kFp8) {
         const int k = 4 * (4 * wave + i) + (lane >> 4);
         const int c = (lane & 15) ^ (2 * (k & 7));
         s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
@@ -332,7 +341,7 @@ struct Gemm256 {
       }
     }
     s.step_a = kStepK * kEsz;
-    s.step_b = (uint32_t)(kStepK * g.ldb * kEsz);
+    s.step_b = kBKMajor ? (uint32_t)(kStepK * kEsz) : (uint32_t)(kStepK * g.ldb * kEsz);
     s.kt_base = 0;
     s.kt_switch = 0x7fffffff;
     s.row0 = row0;
@@ -349,6 +358,13 @@ struct Gemm256 {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + 8 * (4 * wave + i) * kARow256), 16, oa, 0, 0, 0);
   }
   TCCL_D void issue_b(char* stage, const Source& s, int kt, int i) const {
+    if constexpr (kBKMajor) {
+      const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);
+      const bool dead = kt * kStepK + kc * kChunkK >= g.K;
+      const uint32_t ob = dead ? 0xfffffff0u : s.off_b[i] + kt * s.step_b;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + 8 * (4 * wave + i) * kARow256), 16, ob, 0, 0, 0);
+      return;
+    }
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + (4 * wave + i) * 1024), 16,
                                              s.off_b[i] + kt * s.step_b, 0, 0, 0);
   }
@@ -370,7 +386,9 @@ struct Gemm256 {
     Reader r;
     r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
     r.a_swz = (uint32_t)((l32 >> 1) & 7);
-    if constexpr (kFp8) {
+    if constexpr (kBKMajor) {
+      r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + l32) * kARow256);  // this lane's row of column block 0
+    } else if constexpr (kFp8) {
       // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns of k row i/2
       // (column block i%2) and lane j receives 8 consecutive k of column j.  Four reads
       // (k + 0, 8, 16, 24) give the 32 consecutive k of v_mfma_f32_32x32x64_f8f6f4.
@@ -403,6 +421,16 @@ struct Gemm256 {
     return __builtin_bit_cast(Vec, both);
   }
   TCCL_D Vec load_b8(const char* stage, const Reader& r, int kk, int b) const {
+    if constexpr (kBKMajor) {
+      const int half = lane >> 5;
+      const uint32_t chunk = ((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz;
+      const char* row = stage + r.b_base0 + b * 32 * kARow256;
+      const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
+      const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
+      typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+      const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(Vec, both);
+    }
     const char* p = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 32u)) + 64 * kk * kBPitch;
     i32x2 q[4];
 #pragma unroll
@@ -422,6 +450,13 @@ struct Gemm256 {
     return *(const Vec*)(stage + r.a_base + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4) + bi * 32 * kARow256);
   }
   TCCL_D void load_b16(const char* stage, const Reader& r, int kk, Vec (&fb)[2]) const {
+    if constexpr (kBKMajor) {
+      const int half = lane >> 5;
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        fb[b] = *(const Vec*)(stage + r.b_base0 + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4) + b * 32 * kARow256);
+      return;
+    }
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch;
