@@ -253,21 +253,43 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
                      const tccl_heap_view* heap, const tccl_transport_desc* transport,
                      int32_t emulate_peer, void* stream);
 
-/* tccl_allreduce_staged: the staged peer-read all-reduce of the public allreduce launcher
- * (_allreduce_staged_kernel / _allreduce_staged_kernel_ws2, primitives/collectives.py:840-1044;
- * launcher :1882-1946, workspace :2813-2838).  In place on `tensor` (numel elements of `dtype`
- * F16 / BF16 / F32, whole 16-byte units) at the same offset of every rank's slice.  Per chunk of
- * chunk_elems a rank snapshots its values into its `staging` slot, publishes epoch
- * base_epoch + chunk in `published[slot]`, waits for every peer's matching epoch, adds the
- * ranks' values in ascending rank order (fp32 accumulation, one rounding: every rank stores the
- * same bits; the reference starts from its own values and adds in the tensor's type) and
- * acknowledges in the peer's `consumed[slot]`; a rank leaves a slot once world - 1 peers have
- * acknowledged.  staging (slots x chunk_elems), published and consumed
- * (int32[slots], zero before the first call) live in the heap.  `ranks` is the bit mask of the
- * ranks whose roles this launch carries: one process per GPU passes 1 << rank; on one GPU, where
- * the ranks are slices of one arena, all of them run as workgroups of one launch (slots
- * workgroups per rank, all resident).  The caller advances base_epoch by the chunk count per
- * call.  `fault` / `spin_limit_ns` as in tccl_sync_desc. */
+/* tccl_collective_staged: the staged peer-read collectives of the public launchers
+ * (_allreduce_staged_kernel, primitives/collectives.py:840-962, and the two-rank kernels
+ * _allreduce_ / _allgather_ / _reduce_scatter_ / _broadcast_ / _scatter_staged_kernel_ws2,
+ * :966-1592; launchers :1882-2478, workspace :2813-2838), for any world size.  Buffers are given
+ * by rank `heap->rank`'s addresses and sit at the same offset of every rank's slice.
+ *   op              src                      dst                       a block is
+ *   ALLREDUCE       unused (NULL)            the tensor, in place      the tensor
+ *   ALLGATHER       the rank's block         world blocks              src
+ *   REDUCE_SCATTER  world blocks             one block                 dst
+ *   BROADCAST       unused (NULL)            the tensor, in place      the tensor
+ *   SCATTER         world blocks (root's)    one block                 dst
+ * block_elems elements of `dtype` (whole 16-byte units); reductions take F16 / BF16 / F32 and
+ * accumulate in fp32 with one rounding (all-reduce: ranks ascending, the same bits on every rank;
+ * reduce-scatter: the owner's block first, then ranks ascending; the reference adds in the
+ * tensor's type), copies move bytes of any listed dtype.  Per chunk of chunk_elems a publisher
+ * (every rank; BROADCAST / SCATTER: `root`) snapshots what its peers need into its `staging` slot
+ * and stores epoch base_epoch + chunk in `published[slot]`; a consumer waits for that epoch, reads
+ * the slot, writes its own output and adds 1 to the publisher's `consumed[slot]`; the publisher
+ * leaves the slot at world - 1.  staging holds slots x segments x chunk_elems elements (segments
+ * = world for REDUCE_SCATTER and SCATTER, else 1); published and consumed are int32[slots], zero
+ * before the first call; all three live in the heap.  The caller advances base_epoch by the chunk
+ * count per call.  `ranks` is the bit mask of the ranks whose roles this launch carries: one
+ * process per GPU passes 1 << rank; on one GPU, where the ranks are slices of one arena, all of
+ * them run as workgroups of one launch (slots workgroups per rank, all resident).  `fault` /
+ * `spin_limit_ns` as in tccl_sync_desc: a wait that expires raises *fault and ends its role. */
+#define TCCL_STAGED_ALLREDUCE 0
+#define TCCL_STAGED_ALLGATHER 1
+#define TCCL_STAGED_REDUCE_SCATTER 2
+#define TCCL_STAGED_BROADCAST 3
+#define TCCL_STAGED_SCATTER 4
+int tccl_collective_staged(int32_t op, const void* src, void* dst, int32_t dtype, int64_t block_elems, void* staging,
+                           int32_t* published, int32_t* consumed, int32_t chunk_elems, int32_t slots,
+                           int32_t base_epoch, uint32_t ranks, int32_t root, const tccl_heap_view* heap,
+                           int64_t* fault, int64_t spin_limit_ns, void* stream);
+
+/* tccl_allreduce_staged: tccl_collective_staged(TCCL_STAGED_ALLREDUCE, NULL, tensor, ...), the
+ * kernel behind the reference's public allreduce (primitives/collectives.py:1905-1946). */
 int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* staging, int32_t* published,
                           int32_t* consumed, int32_t chunk_elems, int32_t slots, int32_t base_epoch,
                           uint32_t ranks, const tccl_heap_view* heap, int64_t* fault, int64_t spin_limit_ns,

@@ -191,6 +191,136 @@ def test_staged_allreduce_all_roles_in_one_launch(lib, world, numel, dtype, chun
         close(heaps)
 
 
+STAGED_CASES = [
+    # world, block, dtype, chunk_elems, pipeline_slots
+    (2, 1 << 16, torch.float16, None, None),
+    (2, 1 << 19, torch.bfloat16, 4096, 4),       # 128 chunks through 4 slots
+    (3, 40 * 8, torch.float16, 64, 2),           # five chunks, the last one short
+    (4, 3 * 4096 + 4, torch.float32, 4096, None),
+    (8, 4096, torch.float16, 1024, 3),
+    (2, 16, torch.int8, None, None),             # copies move bytes of any 1 / 2 / 4-byte type
+]
+REDUCING = [c for c in STAGED_CASES if c[2] != torch.int8]
+
+
+def staged_inputs(world, shape, dtype, seed):
+    if dtype == torch.int8:
+        g = torch.Generator().manual_seed(seed)
+        return [torch.randint(-128, 127, shape, generator=g, dtype=torch.int8) for _ in range(world)]
+    return [seeded(shape, seed + r, dtype) for r in range(world)]
+
+
+def raw(t):
+    return t.contiguous().view(torch.uint8)
+
+
+@pytest.mark.parametrize("world,block,dtype,chunk,slots", STAGED_CASES)
+def test_staged_allgather(lib, world, block, dtype, chunk, slots):
+    from tileccl_amd.primitives import allgather_staged
+
+    heaps = heaps_of(world)
+    try:
+        for call in range(2):  # the second call reuses the workspace: epochs continue
+            cpu = staged_inputs(world, (block,), dtype, 100 + 10 * call)
+            ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+            outs = [h.allocate_tensor((world * block,), dtype) for h in heaps]
+            for o in outs:
+                raw(o).zero_()
+            fault = allgather_staged(ts, outs, heaps, chunk_elems=chunk, pipeline_slots=slots)
+            torch.cuda.synchronize()
+            assert int(fault.item()) == 0
+            want = oracle.allgather(cpu)
+            for r in range(world):
+                assert torch.equal(raw(outs[r]).cpu(), raw(want[r])), (call, r)
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,block,dtype,chunk,slots", REDUCING)
+def test_staged_reduce_scatter(lib, world, block, dtype, chunk, slots):
+    from tileccl_amd.primitives import reduce_scatter_staged
+
+    heaps = heaps_of(world)
+    try:
+        for call in range(2):
+            cpu = staged_inputs(world, (world * block,), dtype, 200 + 10 * call)
+            ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+            outs = [h.allocate_tensor((block,), dtype) for h in heaps]
+            for o in outs:
+                o.zero_()
+            fault = reduce_scatter_staged(ts, outs, heaps, chunk_elems=chunk, pipeline_slots=slots)
+            torch.cuda.synchronize()
+            assert int(fault.item()) == 0
+            want = oracle.reduce_scatter(cpu, dtype)  # the owner's chunk first, then the other ranks ascending
+            for r in range(world):
+                assert torch.equal(raw(outs[r]).cpu(), raw(want[r])), (call, r)
+                assert torch.equal(raw(ts[r]).cpu(), raw(cpu[r]))  # inputs untouched
+    finally:
+        close(heaps)
+
+
+@pytest.mark.parametrize("world,block,dtype,chunk,slots", STAGED_CASES)
+def test_staged_broadcast_and_scatter(lib, world, block, dtype, chunk, slots):
+    from tileccl_amd.primitives import broadcast_staged, scatter_staged
+
+    heaps = heaps_of(world)
+    try:
+        for root in (0, world - 1):
+            cpu = staged_inputs(world, (block,), dtype, 300 + root)
+            ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+            fault = broadcast_staged(ts, heaps, root=root, chunk_elems=chunk, pipeline_slots=slots)
+            torch.cuda.synchronize()
+            assert int(fault.item()) == 0
+            for r, w in enumerate(oracle.broadcast(cpu, root)):
+                assert torch.equal(raw(ts[r]).cpu(), raw(w)), (root, r)
+
+            full = staged_inputs(world, (world * block,), dtype, 400 + root)
+            srcs = [into_heap(h, c) for h, c in zip(heaps, full)]
+            outs = [h.allocate_tensor((block,), dtype) for h in heaps]
+            for o in outs:
+                raw(o).zero_()
+            fault = scatter_staged(srcs, outs, heaps, root=root, chunk_elems=chunk, pipeline_slots=slots)
+            torch.cuda.synchronize()
+            assert int(fault.item()) == 0
+            for r, w in enumerate(oracle.scatter(full[root], world)):
+                assert torch.equal(raw(outs[r]).cpu(), raw(w)), (root, r)
+    finally:
+        close(heaps)
+
+
+def test_staged_collectives_world_one_and_contracts(lib):
+    from tileccl_amd.primitives import allgather_staged, broadcast_staged, reduce_scatter_staged, scatter_staged
+
+    solo = heaps_of(1)
+    try:
+        t = into_heap(solo[0], seeded((64,), 1))
+        o = solo[0].allocate_tensor((64,), torch.float16)
+        for fn in (allgather_staged, reduce_scatter_staged, scatter_staged):
+            o.zero_()
+            fn([t], [o], solo)
+            torch.cuda.synchronize()
+            assert torch.equal(o, t)
+        broadcast_staged([t], solo)
+    finally:
+        close(solo)
+    heaps = heaps_of(2)
+    try:
+        a = [h.allocate_tensor((64,), torch.float16) for h in heaps]
+        b = [h.allocate_tensor((128,), torch.float16) for h in heaps]
+        with pytest.raises(ValueError, match="allgather output.numel must equal"):
+            allgather_staged(b, a, heaps)
+        with pytest.raises(ValueError, match="root=2 out of range"):
+            broadcast_staged(a, heaps, root=2)
+        with pytest.raises(ValueError, match="reduce_scatter tensor.numel must equal"):
+            reduce_scatter_staged(a, b, heaps)
+        with pytest.raises(ValueError, match="Only op='sum'"):
+            reduce_scatter_staged(b, a, heaps, op="max")
+        with pytest.raises(ValueError, match="one output and one heap per rank"):
+            scatter_staged(b, a[:1], heaps)
+    finally:
+        close(heaps)
+
+
 def test_staged_allreduce_integer_valued_sums_are_exact(lib):
     """A check that does not go through the oracle: small integers add exactly in every order and type."""
     from tileccl_amd.primitives import allreduce_staged

@@ -63,6 +63,7 @@ class GemmDesc(C.Structure):
 
 GEMM_OWN_ROWS_IN_REGISTERS = 1  # TCCL_GEMM_OWN_ROWS_IN_REGISTERS
 GEMM_B_KMAJOR = 2  # TCCL_GEMM_B_KMAJOR
+STAGED_ALLREDUCE, STAGED_ALLGATHER, STAGED_REDUCE_SCATTER, STAGED_BROADCAST, STAGED_SCATTER = range(5)  # TCCL_STAGED_*
 
 
 class SyncDesc(C.Structure):
@@ -144,6 +145,10 @@ SIGNATURES = {
     "tccl_reduce_rows": (
         C.c_int,
         [_vp, _i32, _i64, _vp, _i32, _i64, _i32, _i32, _P(HeapView), _P(TransportDesc), _i32, _vp],
+    ),
+    "tccl_collective_staged": (
+        C.c_int,
+        [_i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _i32, _i32, _i32, C.c_uint32, _i32, _P(HeapView), _vp, _i64, _vp],
     ),
     "tccl_allreduce_staged": (
         C.c_int,

@@ -104,8 +104,8 @@ __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
 }
 
-// Staged all-reduce: workgroup w carries slot w % slots of the (w / slots)-th rank named in a.ranks.
-__global__ __launch_bounds__(256) void staged_allreduce_kernel(tccl::StagedArgs a) {
+// Staged collectives: workgroup w carries slot w % slots of the (w / slots)-th rank named in a.ranks.
+__global__ __launch_bounds__(256) void staged_kernel(tccl::StagedArgs a) {
   __shared__ int word;
   int which = (int)blockIdx.x / a.slots, r = 0;
   for (; r < a.world; ++r)
@@ -1086,29 +1086,40 @@ static int allscatter_impl(const tccl_gemm_desc* d, const tccl_scatter_desc* sc,
   return run_variant(d, c, sync, tr, variant, dev, g, stream, gather, heap);
 }
 
-int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* staging, int32_t* published, int32_t* consumed,
-                          int32_t chunk_elems, int32_t slots, int32_t base_epoch, uint32_t ranks, const tccl_heap_view* heap,
-                          int64_t* fault, int64_t spin_limit_ns, void* stream) {
+int tccl_collective_staged(int32_t op, const void* src, void* dst, int32_t dtype, int64_t block_elems, void* staging,
+                           int32_t* published, int32_t* consumed, int32_t chunk_elems, int32_t slots, int32_t base_epoch,
+                           uint32_t ranks, int32_t root, const tccl_heap_view* heap, int64_t* fault, int64_t spin_limit_ns,
+                           void* stream) {
+  static const char* const names[] = {"allreduce", "allgather", "reduce_scatter", "broadcast", "scatter"};
   int rc = check_heap(heap);
   if (rc) return rc;
+  if (op < TCCL_STAGED_ALLREDUCE || op > TCCL_STAGED_SCATTER) return fail(TCCL_ERR_INVALID, "collective_staged: unknown op %d", op);
+  const char* name = names[op];
+  const bool reduces = op == TCCL_STAGED_ALLREDUCE || op == TCCL_STAGED_REDUCE_SCATTER;
+  const bool in_place = op == TCCL_STAGED_ALLREDUCE || op == TCCL_STAGED_BROADCAST;
+  const bool rooted = op == TCCL_STAGED_BROADCAST || op == TCCL_STAGED_SCATTER;
   const int esize = (int)dtype_size(dtype);
-  if (dtype != TCCL_F16 && dtype != TCCL_BF16 && dtype != TCCL_F32) return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: dtype %d", dtype);
-  if (!tensor || !staging || !published || !consumed || numel <= 0 || chunk_elems <= 0 || slots <= 0 || base_epoch < 1)
-    return fail(TCCL_ERR_INVALID, "allreduce_staged: bad arguments");
+  if (!esize || (reduces && dtype != TCCL_F16 && dtype != TCCL_BF16 && dtype != TCCL_F32))
+    return fail(TCCL_ERR_UNSUPPORTED, "%s_staged: dtype %d", name, dtype);
+  if (!dst || (!in_place && !src) || !staging || !published || !consumed || block_elems <= 0 || chunk_elems <= 0 || slots <= 0 ||
+      base_epoch < 1)
+    return fail(TCCL_ERR_INVALID, "%s_staged: bad arguments", name);
+  if (rooted && (root < 0 || root >= heap->world_size)) return fail(TCCL_ERR_INVALID, "%s_staged: root=%d out of range [0, %d)", name, root, heap->world_size);
   const int per_unit = 16 / esize;
-  if (numel % per_unit || chunk_elems % per_unit || !aligned16(tensor) || !aligned16(staging))
-    return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: tensor and chunk must be whole 16-byte units (%d elements)", per_unit);
-  if ((int64_t)chunk_elems * esize > 0x7fffffffll) return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: chunk too large");
-  if (heap->world_size < 32 && (ranks >> heap->world_size)) return fail(TCCL_ERR_INVALID, "allreduce_staged: ranks=0x%x names ranks beyond world_size=%d", ranks, heap->world_size);
+  if (block_elems % per_unit || chunk_elems % per_unit || !aligned16(dst) || !aligned16(src) || !aligned16(staging))
+    return fail(TCCL_ERR_UNSUPPORTED, "%s_staged: blocks and chunks must be whole 16-byte units (%d elements)", name, per_unit);
+  if ((int64_t)chunk_elems * esize * heap->world_size > 0x7fffffffll) return fail(TCCL_ERR_UNSUPPORTED, "%s_staged: chunk too large", name);
+  if (heap->world_size < 32 && (ranks >> heap->world_size))
+    return fail(TCCL_ERR_INVALID, "%s_staged: ranks=0x%x names ranks beyond world_size=%d", name, ranks, heap->world_size);
   const int roles = __builtin_popcount(ranks);
   if (roles == 0) return 0;
-  const int64_t chunks = (numel + chunk_elems - 1) / chunk_elems;
-  if ((int64_t)base_epoch + chunks > 0x7fffffffll) return fail(TCCL_ERR_INVALID, "allreduce_staged: epoch range overflows int32");
+  const int64_t chunks = (block_elems + chunk_elems - 1) / chunk_elems;
+  if ((int64_t)base_epoch + chunks > 0x7fffffffll) return fail(TCCL_ERR_INVALID, "%s_staged: epoch range overflows int32", name);
   tccl_device_info dev;
   if ((rc = query_device(-1, &dev))) return rc;
   // Every (rank, slot) workgroup waits on others of the same launch: all must be resident.
   if ((int64_t)roles * slots > (int64_t)dev.compute_units * 4)
-    return fail(TCCL_ERR_UNSUPPORTED, "allreduce_staged: %d roles x %d slots exceed what the device keeps resident (%d workgroups)", roles,
+    return fail(TCCL_ERR_UNSUPPORTED, "%s_staged: %d roles x %d slots exceed what the device keeps resident (%d workgroups)", name, roles,
                 slots, dev.compute_units * 4);
   tccl::StagedArgs a;
   memset(&a, 0, sizeof a);
@@ -1116,20 +1127,30 @@ int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* stag
   a.rank = heap->rank;
   a.world = heap->world_size;
   a.ranks = ranks;
-  a.tensor = (char*)tensor;
+  a.op = op;
+  a.root = root;
+  a.src = (char*)src;
+  a.dst = (char*)dst;
   a.staging = (char*)staging;
   a.published = published;
   a.consumed = consumed;
-  a.units = numel / per_unit;
+  a.units = block_elems / per_unit;
   a.chunk_units = chunk_elems / per_unit;
   a.slots = slots;
   a.base_epoch = base_epoch;
-  a.dtype = dtype;
+  a.dtype = reduces ? dtype : TCCL_F16;  // copies move bytes
   a.fault = fault;
   a.spin_ticks = (spin_limit_ns > 0 ? spin_limit_ns : kDefaultSpinNs) / 10 + 1;
-  hipLaunchKernelGGL(staged_allreduce_kernel, dim3(roles * slots), dim3(256), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(staged_kernel, dim3(roles * slots), dim3(256), 0, (hipStream_t)stream, a);
   TCCL_HIP(hipGetLastError());
   return 0;
+}
+
+int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* staging, int32_t* published, int32_t* consumed,
+                          int32_t chunk_elems, int32_t slots, int32_t base_epoch, uint32_t ranks, const tccl_heap_view* heap,
+                          int64_t* fault, int64_t spin_limit_ns, void* stream) {
+  return tccl_collective_staged(TCCL_STAGED_ALLREDUCE, nullptr, tensor, dtype, numel, staging, published, consumed, chunk_elems, slots,
+                                base_epoch, ranks, 0, heap, fault, spin_limit_ns, stream);
 }
 
 int tccl_gemm_allscatter(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,

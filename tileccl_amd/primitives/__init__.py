@@ -5,7 +5,11 @@ from tileccl_amd.primitives.collectives import (
     MAX_COLLECTIVE_WORLD_SIZE,
     allgather,
     allreduce,
+    allgather_staged,
     allreduce_staged,
+    broadcast_staged,
+    reduce_scatter_staged,
+    scatter_staged,
     broadcast,
     reduce_scatter,
     scatter,
@@ -16,7 +20,11 @@ __all__ = [
     "MAX_COLLECTIVE_WORLD_SIZE",
     "allgather",
     "allreduce",
+    "allgather_staged",
     "allreduce_staged",
+    "broadcast_staged",
+    "reduce_scatter_staged",
+    "scatter_staged",
     "broadcast",
     "copy_block",
     "get",

@@ -5,10 +5,9 @@ reduce_scatter`` (``/root/reference/tileccl/primitives/collectives.py:1882-2478`
 same argument order, contracts and messages.  The data movement is the reference's
 direct-write / peer-read form (``tile_allgather`` :613-663, ``tile_scatter`` :671-727,
 ``tile_reduce_scatter`` :730-783, ``tile_broadcast`` :791-836) on this package's bulk copy and
-reduce kernels.  Its staged peer-read all-reduce (:840-1044: snapshot a chunk, publish an
-epoch, read the peers' snapshots, acknowledge) is ``allreduce_staged``; the other staged
-variants (:1048-1592) are the same slot protocol around the copies above and have no
-counterpart here.
+reduce kernels.  Its staged peer-read kernels (:840-1592: snapshot a chunk into a slot,
+publish an epoch, read the peers' slots, acknowledge) are the ``*_staged`` functions below,
+all roles of a call in one launch.
 
 What differs, on purpose:
 
@@ -222,9 +221,9 @@ def allreduce(tensor: torch.Tensor, heap, op: str = "sum") -> None:
 
 
 # ---------------------------------------------------------------------------------------------
-# The staged peer-read all-reduce (reference :840-1044, launcher :1882-1946).
+# The staged peer-read collectives (reference :840-1592; launchers :1882-2478).
 #
-# A rank's role waits, inside the kernel, for every peer's role of the same call, so the roles
+# A rank's role waits, inside the kernel, for its peers' roles of the same call, so the roles
 # cannot run one call after the other as the collectives above do.  With the ranks emulated as
 # slices of one arena, one launch carries all of them ((rank, slot) -> workgroup); a process
 # that owns a single rank of a real multi-GPU job would pass ``ranks=(heap.rank,)``.
@@ -234,20 +233,21 @@ STAGED_MAX_CHUNK_BYTES = 64 << 10      # ... to 16 x 16 bytes
 STAGED_RESIDENT_WORKGROUPS = 1024      # world x slots must be resident at once (4 workgroups on each of 256 CUs)
 STAGED_MAX_PIPELINE_SLOTS = 256        # workgroups per rank
 _DEFAULT_SPIN_NS = 0                   # the library's default bound on a wait
+_BYTES_AS = {1: torch.float8_e4m3fn, 2: torch.float16, 4: torch.float32}  # a library dtype of each element size
 
 
 class _StagedWorkspace:
     """Staging rows and the two words per slot, at one offset in every rank's slice, plus the
     epoch counter of the calls that used them (reference ``_AllReduceWorkspace``, :2813-2838)."""
 
-    def __init__(self, heaps, dtype: torch.dtype, chunk_elems: int, slots: int) -> None:
-        self.staging = [h.allocate_tensor((slots, chunk_elems), dtype) for h in heaps]
+    def __init__(self, heaps, dtype: torch.dtype, chunk_elems: int, slots: int, segments: int) -> None:
+        self.staging = [h.allocate_tensor((slots, segments, chunk_elems), dtype) for h in heaps]
         self.published = [h.allocate_tensor((slots,), torch.int32) for h in heaps]
         self.consumed = [h.allocate_tensor((slots,), torch.int32) for h in heaps]
         for group in (self.staging, self.published, self.consumed):
             offsets = {h.get_offset(int(t.data_ptr())) for h, t in zip(heaps, group)}
             if len(offsets) != 1:
-                raise RuntimeError("allreduce_staged: the ranks' heaps have diverged, no common workspace offset")
+                raise RuntimeError("staged collective: the ranks' heaps have diverged, no common workspace offset")
         for t in self.published + self.consumed:
             t.zero_()
         self.fault = torch.zeros(1, dtype=torch.int64, device=self.staging[0].device)
@@ -262,17 +262,17 @@ class _StagedWorkspace:
         return base
 
 
-_STAGED: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()  # heap of rank 0 -> {(dtype, chunk, slots): workspace}
+_STAGED: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()  # heap of rank 0 -> {(dtype, chunk, slots, segments): workspace}
 
 
 def resolve_staged_execution(numel: int, element_size: int, world: int, *, chunk_elems: int | None = None,
                              pipeline_slots: int | None = None) -> tuple[int, int, int]:
-    """(chunk_elems, chunks, pipeline_slots) for a tensor: as many slots as stay resident, at
-    most 256 per rank, and the smallest chunk of 16 / 32 / 64 KiB that gives every slot work
-    (measured on two and four ranks, 1 MiB to 256 MiB: more slots always won; 16 KiB chunks
-    are quickest while the slots outnumber them, 64 KiB chunks from there on).  The reference's
-    policy (:2586-2597) picks 256..4096 elements and at most 16 programs for its target; the
-    contract is the same."""
+    """(chunk_elems, chunks, pipeline_slots) for a block of ``numel`` elements: as many slots as
+    stay resident, at most 256 per rank, and the smallest chunk of 16 / 32 / 64 KiB that gives
+    every slot work (measured for the all-reduce on two and four ranks, 1 MiB to 256 MiB: more
+    slots always won; 16 KiB chunks are quickest while the slots outnumber them, 64 KiB chunks
+    from there on).  The reference's policy (:2586-2597, :1802-1880) picks 256..4096 elements and
+    at most 8 or 16 programs for its target; the contract is the same."""
     per_unit = 16 // element_size
     slot_cap = max(1, min(STAGED_MAX_PIPELINE_SLOTS, STAGED_RESIDENT_WORKGROUPS // world))
     if chunk_elems is None:
@@ -281,53 +281,49 @@ def resolve_staged_execution(numel: int, element_size: int, world: int, *, chunk
             chunk_bytes *= 2
         chunk_elems = min(chunk_bytes // element_size, -(-numel // per_unit) * per_unit)
     if chunk_elems <= 0 or chunk_elems % per_unit:
-        raise ValueError(f"allreduce_staged: chunk_elems={chunk_elems} must be a positive multiple of {per_unit}")
+        raise ValueError(f"staged collective: chunk_elems={chunk_elems} must be a positive multiple of {per_unit}")
     chunks = -(-numel // chunk_elems)
     if pipeline_slots is None:
         pipeline_slots = min(chunks, slot_cap)
     if pipeline_slots < 1:
-        raise ValueError(f"allreduce_staged: pipeline_slots={pipeline_slots} must be at least 1")
+        raise ValueError(f"staged collective: pipeline_slots={pipeline_slots} must be at least 1")
     return chunk_elems, chunks, min(pipeline_slots, chunks)
 
 
-def allreduce_staged(tensors, heaps, op: str = "sum", *, chunk_elems: int | None = None, pipeline_slots: int | None = None,
-                     ranks=None, spin_limit_ns: int = _DEFAULT_SPIN_NS) -> torch.Tensor:
-    """In place on every rank's tensor, in one launch: each ends with the sum over ranks.
-
-    ``tensors[r]`` is rank ``r``'s tensor in ``heaps[r]``, all at one heap offset.  ``ranks``
-    names the roles the launch carries (default: all).  Returns the fault word of the
-    workspace (int64[1] on the device): non-zero after a wait ran into ``spin_limit_ns``,
-    which is what happens when a role that the others wait for is left out.
-    """
-    if op != "sum":
-        raise ValueError(f"Only op='sum' is currently supported, got {op!r}")
+def _one_per_rank(name: str, what: str, tensors, heaps) -> None:
     world = len(heaps)
     if len(tensors) != world or any(h.world_size != world or h.rank != r for r, h in enumerate(heaps)):
-        raise ValueError("allreduce_staged expects one tensor and one heap per rank, in rank order")
-    _validate_world_size(world)
+        raise ValueError(f"{name} expects one {what} and one heap per rank, in rank order")
     first = tensors[0]
     for r, (t, h) in enumerate(zip(tensors, heaps)):
-        _contiguous("allreduce_staged", t, f"tensors[{r}]")
-        _on_heap(t, h, f"tensors[{r}]")
+        _contiguous(name, t, f"{what}s[{r}]")
+        _on_heap(t, h, f"{what}s[{r}]")
         if t.dtype != first.dtype or t.shape != first.shape:
-            raise ValueError("allreduce_staged expects one dtype and shape on every rank")
+            raise ValueError(f"{name} expects one dtype and shape on every rank")
     if len({h.get_offset(int(t.data_ptr())) for t, h in zip(tensors, heaps)}) != 1:
-        raise ValueError("allreduce_staged expects the tensor at the same heap offset on every rank")
-    if first.dtype not in _REDUCE_IN:
-        raise ValueError(f"allreduce_staged supports fp16, bf16 and fp32 tensors, got {first.dtype}")
-    numel = int(first.numel())
+        raise ValueError(f"{name} expects the {what} at the same heap offset on every rank")
+
+
+def _staged(name: str, op: int, srcs, dsts, heaps, block: int, *, root: int = 0, chunk_elems=None, pipeline_slots=None,
+            ranks=None, spin_limit_ns: int = _DEFAULT_SPIN_NS) -> torch.Tensor:
+    """One launch of ``tccl_collective_staged`` with the roles of ``ranks`` (default: every rank).
+    Returns the workspace's fault word (int64[1] on the device): non-zero after a wait ran into
+    ``spin_limit_ns``, which is what happens when a role that the others wait for is left out."""
+    world = len(heaps)
+    first = dsts[0]
     carried = tuple(range(world)) if ranks is None else tuple(int(r) for r in ranks)
     for r in carried:
         _validate_root(r, world_size=world)
+    if world == 1 or block == 0 or not carried:
+        return torch.zeros(1, dtype=torch.int64, device=first.device)
+    esz = first.element_size()
+    _whole_units(name, block, esz)
+    chunk_elems, chunks, slots = resolve_staged_execution(block, esz, world, chunk_elems=chunk_elems, pipeline_slots=pipeline_slots)
+    segments = world if op in (_lib.STAGED_REDUCE_SCATTER, _lib.STAGED_SCATTER) else 1
     cache = _STAGED.setdefault(heaps[0], {})
-    if world == 1 or numel == 0 or not carried:
-        return torch.zeros(1, dtype=torch.int64, device=first.device)  # local identity (reference :2563-2583)
-    _whole_units("allreduce_staged", numel, first.element_size())
-    chunk_elems, chunks, slots = resolve_staged_execution(numel, first.element_size(), world, chunk_elems=chunk_elems,
-                                                          pipeline_slots=pipeline_slots)
-    key = (str(first.dtype), chunk_elems, slots)
+    key = (str(first.dtype), chunk_elems, slots, segments)
     if key not in cache:
-        cache[key] = _StagedWorkspace(heaps, first.dtype, chunk_elems, slots)
+        cache[key] = _StagedWorkspace(heaps, first.dtype, chunk_elems, slots, segments)
     ws = cache[key]
     base_epoch = ws.reserve_epoch_range(chunks)
     ws.fault.zero_()
@@ -335,10 +331,82 @@ def allreduce_staged(tensors, heaps, op: str = "sum", *, chunk_elems: int | None
     mask = 0
     for r in carried:
         mask |= 1 << r
-    rc = _lib.load().tccl_allreduce_staged(
-        _launch.ptr(tensors[0]), _launch.dtype_code(first.dtype), numel, _launch.ptr(ws.staging[0]), _launch.ptr(ws.published[0]),
-        _launch.ptr(ws.consumed[0]), chunk_elems, slots, base_epoch, mask, _launch.byref(view), _launch.ptr(ws.fault),
-        int(spin_limit_ns), _launch.stream_ptr(),
+    reduces = op in (_lib.STAGED_ALLREDUCE, _lib.STAGED_REDUCE_SCATTER)
+    code = _launch.dtype_code(first.dtype if reduces else _BYTES_AS.get(esz, first.dtype))  # copies move bytes
+    rc = _lib.load().tccl_collective_staged(
+        op, _launch.ptr(srcs[0]) if srcs is not None else None, _launch.ptr(dsts[0]), code, block,
+        _launch.ptr(ws.staging[0]), _launch.ptr(ws.published[0]), _launch.ptr(ws.consumed[0]), chunk_elems, slots, base_epoch, mask,
+        int(root), _launch.byref(view), _launch.ptr(ws.fault), int(spin_limit_ns), _launch.stream_ptr(),
     )
-    _lib.check(rc, "tccl_allreduce_staged")
+    _lib.check(rc, f"tccl_collective_staged[{name}]")
     return ws.fault
+
+
+def allreduce_staged(tensors, heaps, op: str = "sum", **how) -> torch.Tensor:
+    """In place on every rank's tensor, in one launch: each ends with the sum over ranks (the ranks'
+    values added in ascending rank order in fp32, one rounding: the same bits everywhere).
+    ``tensors[r]`` is rank ``r``'s tensor in ``heaps[r]``, all at one heap offset.  Keywords
+    ``chunk_elems``, ``pipeline_slots``, ``ranks``, ``spin_limit_ns``: see ``_staged``."""
+    if op != "sum":
+        raise ValueError(f"Only op='sum' is currently supported, got {op!r}")
+    _validate_world_size(len(heaps))
+    _one_per_rank("allreduce_staged", "tensor", tensors, heaps)
+    if tensors[0].dtype not in _REDUCE_IN:
+        raise ValueError(f"allreduce_staged supports fp16, bf16 and fp32 tensors, got {tensors[0].dtype}")
+    return _staged("allreduce_staged", _lib.STAGED_ALLREDUCE, None, tensors, heaps, int(tensors[0].numel()), **how)
+
+
+def allgather_staged(tensors, outputs, heaps, **how) -> torch.Tensor:
+    """Every rank's ``output`` ends with ``[tensor_rank0 | tensor_rank1 | ...]`` (reference :1129-1215)."""
+    world = len(heaps)
+    _validate_world_size(world)
+    _one_per_rank("allgather_staged", "tensor", tensors, heaps)
+    _one_per_rank("allgather_staged", "output", outputs, heaps)
+    block = _pair_block("allgather", tensor=tensors[0], output=outputs[0], world_size=world)
+    if tensors[0].dtype != outputs[0].dtype:
+        raise ValueError(f"allgather expects one dtype, got tensor={tensors[0].dtype}, output={outputs[0].dtype}")
+    if world == 1 and block:
+        outputs[0].reshape(-1).copy_(tensors[0].reshape(-1))
+    return _staged("allgather_staged", _lib.STAGED_ALLGATHER, tensors, outputs, heaps, block, **how)
+
+
+def reduce_scatter_staged(tensors, outputs, heaps, op: str = "sum", **how) -> torch.Tensor:
+    """Rank ``r``'s ``output`` = its own chunk ``r`` plus the other ranks' chunk ``r`` in ascending rank
+    (fp32 accumulation, one rounding; reference :1276-1366 and tile_reduce_scatter's order :766-781)."""
+    if op != "sum":
+        raise ValueError(f"Only op='sum' is currently supported, got {op!r}")
+    world = len(heaps)
+    _validate_world_size(world)
+    _one_per_rank("reduce_scatter_staged", "tensor", tensors, heaps)
+    _one_per_rank("reduce_scatter_staged", "output", outputs, heaps)
+    block = _pair_block("reduce_scatter", tensor=tensors[0], output=outputs[0], world_size=world)
+    if tensors[0].dtype not in _REDUCE_IN or outputs[0].dtype != tensors[0].dtype:
+        raise ValueError(f"reduce_scatter_staged supports fp16, bf16 and fp32, output of the tensor's type; got "
+                         f"{tensors[0].dtype} -> {outputs[0].dtype}")
+    if world == 1 and block:
+        outputs[0].reshape(-1).copy_(tensors[0].reshape(-1))
+    return _staged("reduce_scatter_staged", _lib.STAGED_REDUCE_SCATTER, tensors, outputs, heaps, block, **how)
+
+
+def broadcast_staged(tensors, heaps, root: int = 0, **how) -> torch.Tensor:
+    """Every rank's tensor ends with the root's (reference :1391-1486)."""
+    world = len(heaps)
+    _validate_world_size(world)
+    _validate_root(root, world_size=world)
+    _one_per_rank("broadcast_staged", "tensor", tensors, heaps)
+    return _staged("broadcast_staged", _lib.STAGED_BROADCAST, None, tensors, heaps, int(tensors[0].numel()), root=root, **how)
+
+
+def scatter_staged(tensors, outputs, heaps, *, root: int = 0, **how) -> torch.Tensor:
+    """Rank ``i``'s ``output`` receives chunk ``i`` of the root's ``tensor`` (reference :1489-1592)."""
+    world = len(heaps)
+    _validate_world_size(world)
+    _validate_root(root, world_size=world)
+    _one_per_rank("scatter_staged", "tensor", tensors, heaps)
+    _one_per_rank("scatter_staged", "output", outputs, heaps)
+    block = _pair_block("scatter", tensor=tensors[0], output=outputs[0], world_size=world)
+    if tensors[0].dtype != outputs[0].dtype:
+        raise ValueError(f"scatter expects one dtype, got tensor={tensors[0].dtype}, output={outputs[0].dtype}")
+    if world == 1 and block:
+        outputs[0].reshape(-1).copy_(tensors[0].reshape(-1))
+    return _staged("scatter_staged", _lib.STAGED_SCATTER, tensors, outputs, heaps, block, root=root, **how)
