@@ -26,6 +26,7 @@ FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
+    "-fvisibility=hidden",
     "-Wno-comment",
     # hipcc -O3 must not form packed-fp32 instructions on this hardware pool.
     "-Xclang",

@@ -8,7 +8,10 @@
 #include <mutex>
 #include <type_traits>
 
+// The library is built with -fvisibility=hidden: only what the public header declares is exported.
+#pragma GCC visibility push(default)
 #include "../../include/tileccl_hip.h"
+#pragma GCC visibility pop
 #include "tccl_comm.h"
 #include "tccl_gemm.h"
 #include "tccl_gemm256.h"

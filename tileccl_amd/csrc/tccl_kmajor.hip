@@ -5,12 +5,12 @@
 
 namespace tccl {
 
-__attribute__((visibility("hidden"))) int launch_gemm256_kmajor(int in_dtype, int out_dtype, const GemmArgs& g, const Macro& m, int wgs,
+int launch_gemm256_kmajor(int in_dtype, int out_dtype, const GemmArgs& g, const Macro& m, int wgs,
                                                                 hipStream_t stream) {
   return launch_gemm256_table<true>(in_dtype, out_dtype, g, m, wgs, stream);
 }
 
-__attribute__((visibility("hidden"))) int launch_fused256_kmajor(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
+int launch_fused256_kmajor(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
                                                                  hipStream_t stream) {
   return launch_fused256_table<true>(in_dtype, out_dtype, f, wgs, stream);
 }
