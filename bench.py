@@ -271,6 +271,19 @@ class Workload:
         lib = _lib.load()
         return lambda _variant: _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
 
+    def library_gemm(self):
+        """The same GEMM by torch.matmul (the vendor's GEMM library), for context: B row-major as the
+        configurations hold it, and B k-major, the layout that library is fastest with.  16-bit inputs only."""
+        import torch
+
+        if self.in_type == "f8":
+            return None
+        A = self.A.clone()
+        B_kn = self.B.clone() if self.b_layout == "kn" else self.B.t().contiguous().t().contiguous()
+        B_nk = B_kn.t().contiguous()
+        out = torch.empty(self.M, self.N, dtype=A.dtype, device=A.device)
+        return {"kn": lambda _v: torch.matmul(A, B_kn, out=out), "nk": lambda _v: torch.matmul(A, B_nk.t(), out=out)}
+
     def cpu_baseline(self, iters=3):
         """The oracle's restatement of the same operation on the host cores (reported, not a target)."""
         import torch
@@ -452,6 +465,14 @@ def main() -> int:
                      "note": w.one_direction_note}
     _, gemm_mean = time_variant(w.gemm_only(), "s0", args.steps, args.warmup)  # GEMM alone, for the phase split
 
+    library = None
+    if getattr(w, "library_gemm", None) and w.library_gemm():
+        library = {"note": "torch.matmul (vendor GEMM library) on the same operands, for context: B row-major / B k-major"}
+        for layout, run in w.library_gemm().items():
+            _, ms = time_variant(run, "s0", args.steps, args.warmup)
+            library[f"b_{layout}_ms"] = round(ms, 5)
+            library[f"b_{layout}_tflops"] = round(w.flop / (ms * 1e-3) / 1e12, 2)
+
     peak = PEAK_TFLOPS[w.in_type]
     chosen = results[args.variant]
     tflops = chosen["tflops"]  # per launch, HIP events on the launch stream
@@ -499,6 +520,8 @@ def main() -> int:
         line["config"]["b_layout"] = "B held as (N, K), passed as its .t() view"
     if push_only is not None:
         line["one_direction"] = push_only
+    if library is not None:
+        line["library_gemm"] = library
     if "s0" in results and "s2" in results:
         line["s2_vs_s0_speedup"] = round(results["s0"]["event_ms_mean"] / results["s2"]["event_ms_mean"], 4)
     if "s0" in results:
