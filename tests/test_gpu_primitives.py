@@ -288,6 +288,65 @@ def test_staged_broadcast_and_scatter(lib, world, block, dtype, chunk, slots):
         close(heaps)
 
 
+@pytest.mark.parametrize("seed", [21, 22])
+def test_staged_collectives_random_sizes(lib, seed):
+    """Seeded random worlds, block sizes, chunk sizes and slot counts through the five staged
+    collectives, several calls on one set of heaps (workspaces and epochs are reused)."""
+    import random
+
+    from tileccl_amd import primitives as prim
+
+    rng = random.Random(seed)
+    for _ in range(12):
+        world = rng.choice([2, 3, 4, 5, 8])
+        heaps = heaps_of(world, 32 << 20)
+        try:
+            for call in range(6):
+                dtype = rng.choice([torch.float16, torch.bfloat16, torch.float32])
+                per_unit = 16 // (2 if dtype != torch.float32 else 4)
+                block = per_unit * rng.randint(1, 3000)
+                chunk = rng.choice([None, per_unit * rng.randint(1, 400)])
+                slots = rng.choice([None, rng.randint(1, 9)])
+                how = dict(chunk_elems=chunk, pipeline_slots=slots)
+                op = rng.choice(["allreduce", "allgather", "reduce_scatter", "broadcast", "scatter"])
+                root = rng.randrange(world)
+                tag = (seed, world, call, op, dtype, block, chunk, slots, root)
+                if op == "allreduce":
+                    cpu = [seeded((block,), 7 * call + r, dtype) for r in range(world)]
+                    ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+                    fault = prim.allreduce_staged(ts, heaps, **how)
+                    want, got = oracle.allreduce_staged(cpu), ts
+                elif op == "allgather":
+                    cpu = [seeded((block,), 7 * call + r, dtype) for r in range(world)]
+                    ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+                    got = [h.allocate_tensor((world * block,), dtype) for h in heaps]
+                    fault = prim.allgather_staged(ts, got, heaps, **how)
+                    want = oracle.allgather(cpu)
+                elif op == "reduce_scatter":
+                    cpu = [seeded((world * block,), 7 * call + r, dtype) for r in range(world)]
+                    ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+                    got = [h.allocate_tensor((block,), dtype) for h in heaps]
+                    fault = prim.reduce_scatter_staged(ts, got, heaps, **how)
+                    want = oracle.reduce_scatter(cpu, dtype)
+                elif op == "broadcast":
+                    cpu = [seeded((block,), 7 * call + r, dtype) for r in range(world)]
+                    got = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+                    fault = prim.broadcast_staged(got, heaps, root=root, **how)
+                    want = oracle.broadcast(cpu, root)
+                else:
+                    cpu = [seeded((world * block,), 7 * call + r, dtype) for r in range(world)]
+                    ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
+                    got = [h.allocate_tensor((block,), dtype) for h in heaps]
+                    fault = prim.scatter_staged(ts, got, heaps, root=root, **how)
+                    want = oracle.scatter(cpu[root], world)
+                torch.cuda.synchronize()
+                assert int(fault.item()) == 0, tag
+                for r in range(world):
+                    assert torch.equal(raw(got[r]).cpu(), raw(want[r])), (tag, r)
+        finally:
+            close(heaps)
+
+
 def test_staged_collectives_world_one_and_contracts(lib):
     from tileccl_amd.primitives import allgather_staged, broadcast_staged, reduce_scatter_staged, scatter_staged
 
