@@ -97,6 +97,27 @@ def test_ragged_rows_three_ranks_bf16(lib, pattern):
     _two_rank_case(pattern, 200, 72, 384, dtype=torch.bfloat16, world=3)
 
 
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_shapes_every_pattern(lib, seed):
+    """Seeded random shapes, worlds and TileGroup sizes through the full / full contract of every pattern."""
+    import random
+
+    rng = random.Random(seed)
+    for _ in range(40):
+        pattern = rng.choice(PATTERNS)
+        world = rng.choice([1, 2, 3, 4])
+        M, K = rng.randint(1, 1100), 8 * rng.randint(1, 48)
+        N = 8 * world * rng.randint(1, 40)  # the full / full contract splits N over the ranks
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        kw = {}
+        if pattern == "tile_group":
+            kw = dict(tau_min_bytes=rng.choice([1, 1 << 16, 1 << 18]), GROUP_M=rng.choice([1, 2, 8]))
+        try:
+            _two_rank_case(pattern, M, K, N, dtype=dtype, world=world, **kw)
+        except AssertionError as e:
+            raise AssertionError(f"{pattern} world {world} M {M} K {K} N {N} {dtype} {kw}: {e}") from e
+
+
 def test_tile_group_counters_and_many_groups(lib):
     def inspect(plans):
         impl = plans[0].pattern_impl
