@@ -20,7 +20,8 @@ def test_readme_example_runs(lib):
     op, A2, B2 = scope["op"], scope["A2"], scope["B2"]
     op.check_faults()
     assert tuple(op.out.shape) == (8192, 4096)
-    for h in scope["heaps"]:
+    assert all(bool((x == 2.0).all()) for x in scope["xs"])
+    for h in scope["heaps"] + scope["ranks"]:
         h.cleanup()
     for c in scope["ctxs"]:
         c.heap.cleanup()
