@@ -153,6 +153,32 @@ def test_repeated_launches_reuse_unreset_counters(lib):
             c.heap.cleanup()
 
 
+@pytest.mark.parametrize("pattern", ["auto", "bulk_sync", "wg_specialized", "tile_group", "s2"])
+def test_patterns_named_by_string_take_heap_memory_once(lib, pattern):
+    """A pattern given by name is instantiated on every call; its signal words are cut from the heap, which
+    never gives memory back, so they must be found again instead of allocated again."""
+    import tileccl_amd as tileccl
+
+    ctxs = tileccl.init_local(world_size=2, heap_size=64 << 20)
+    try:
+        c = ctxs[0]
+        A = c.as_symmetric(seeded((256, 64), 0).cuda())
+        B = c.as_symmetric(seeded((64, 256), 1, scale=1 / 8).cuda())
+        out = c.zeros(256, 256, dtype=torch.float16)
+        ctxs[1].zeros(256 * 3, 256, dtype=torch.float16)  # the peer's slice is written at the same offsets
+        tileccl.ops.gemm_allscatter(A, B, out, ctx=c, pattern=pattern)
+        used = c.heap.bytes_allocated
+        first = out.clone()
+        for _ in range(20):
+            tileccl.ops.gemm_allscatter(A, B, out, ctx=c, pattern=pattern)
+        torch.cuda.synchronize()
+        assert c.heap.bytes_allocated == used
+        assert torch.equal(bits(out), bits(first))
+    finally:
+        for x in ctxs:
+            x.heap.cleanup()
+
+
 def test_sharded_and_mixed_contracts(lib):
     import tileccl_amd as tileccl
     from tileccl_amd import ops

@@ -33,7 +33,15 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise ValueError(f"dtype {dtype} is not supported by the HIP kernels") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr() -> int:
+    """torch's current stream on the heap's device as a ``hipStream_t`` value.  The raw accessor
+    costs well under a microsecond; building a ``torch.cuda.Stream`` object costs ~9 us, a fifth
+    of a c1-sized launch."""
+    if _raw_stream is not None:
+        return int(_raw_stream(0))  # every emulated rank lives on device 0
     return int(torch.cuda.current_stream().cuda_stream)
 
 

@@ -41,7 +41,12 @@ class _HipAllScatterPattern(Pattern):
             raise ValueError(f"BLOCK_M x BLOCK_N = {BLOCK_M} x {BLOCK_N} must be multiples of 128")
         self.BLOCK_M, self.BLOCK_N, self.BLOCK_K, self.GROUP_M = BLOCK_M, BLOCK_N, BLOCK_K, GROUP_M
         self.NUM_SMS, self.COMPUTE_SMS, self.COMM_SMS = NUM_SMS, COMPUTE_SMS, COMM_SMS
-        self._sync: dict[tuple, _launch.SyncWords] = {}
+        # Signal words are cut from the heap, which never gives memory back, and a pattern named
+        # by a string is instantiated anew on every call (ops._resolve_pattern_impl, as in the
+        # reference, ops.py:1289-1296): they are therefore kept with the context, next to its
+        # workspaces, and shared by every pattern instance of the same kind and tiling.
+        cache = getattr(ctx, "_workspace_cache", None)
+        self._sync: dict[tuple, _launch.SyncWords] = cache if isinstance(cache, dict) else {}
 
     # -- hooks -------------------------------------------------------------------------
     def _sync_words(self, M: int, N: int, C_out: torch.Tensor) -> _launch.SyncWords | None:
@@ -137,7 +142,7 @@ class WGSpecializedPattern(_HipAllScatterPattern):
 
     def _sync_words(self, M: int, N: int, C_out: torch.Tensor) -> _launch.SyncWords:
         tiles = -(-M // self.BLOCK_M) * -(-N // self.BLOCK_N)
-        key = ("locks", tiles)
+        key = ("tileccl_amd.sync", "locks", tiles)
         words = self._sync.get(key)
         if words is None:
             heap = self.ctx.require_heap()
@@ -194,7 +199,8 @@ class TileGroupPattern(_HipAllScatterPattern):
         )
 
     def _sync_words(self, M: int, N: int, C_out: torch.Tensor) -> _launch.SyncWords:
-        key = ("groups", M, N, C_out.element_size())
+        key = ("tileccl_amd.sync", "groups", M, N, C_out.element_size(), self.BLOCK_M, self.BLOCK_N, self.GROUP_M,
+               self.target_group_tiles, self.tau_min_bytes, self.max_groups)
         words = self._sync.get(key)
         if words is None:
             plan = self.plan_for(M, N, C_out.element_size())
