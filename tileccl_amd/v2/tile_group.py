@@ -60,47 +60,26 @@ class TileGroupPlan:
     tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES
     p0_min_tiles: int = 1
 
-    # -- scalar summaries -------------------------------------------------
-    @property
-    def n_groups(self) -> int:
-        return len(self.groups)
+    # -- scalar summaries ----------------------------------------------------
+    n_groups = property(lambda self: len(self.groups))
+    # largest number of tile rows any group spans (row_end not clamped to M), and tile columns of the output
+    max_rb = property(lambda self: max(_cdiv(end - first, self.block_m) for first, end, _ in self.groups))
+    max_cb = property(lambda self: _cdiv(self.N, self.block_n))
+    # largest group payload in elements; row_end is not clamped to M
+    max_group_elems = property(lambda self: max((end - first) * self.N for first, end, _ in self.groups))
+    min_group_tiles = property(lambda self: min(self.tile_counts()))
+    max_group_tiles = property(lambda self: max(self.tile_counts()))
+    avg_group_tiles = property(lambda self: sum(self.tile_counts()) / len(self.groups))
 
-    @property
-    def max_rb(self) -> int:
-        """Largest number of tile rows any group spans (unclamped row_end)."""
-        return max(_cdiv(hi - lo, self.block_m) for lo, hi, _ in self.groups)
+    # -- per-group vectors (what the kernels take) ----------------------------
+    def row_starts(self) -> "list[int]":
+        return [first for first, _, _ in self.groups]
 
-    @property
-    def max_cb(self) -> int:
-        """Tile columns of the output."""
-        return _cdiv(self.N, self.block_n)
+    def row_ends(self) -> "list[int]":
+        return [min(end, self.M) for _, end, _ in self.groups]
 
-    @property
-    def max_group_elems(self) -> int:
-        """Largest group payload in elements; ``row_end`` is not clamped to ``M``."""
-        return max((hi - lo) * self.N for lo, hi, _ in self.groups)
-
-    @property
-    def min_group_tiles(self) -> int:
-        return min(g[2] for g in self.groups)
-
-    @property
-    def max_group_tiles(self) -> int:
-        return max(g[2] for g in self.groups)
-
-    @property
-    def avg_group_tiles(self) -> float:
-        return sum(g[2] for g in self.groups) / len(self.groups)
-
-    # -- per-group vectors (what the kernels take) --------------------------
-    def row_starts(self) -> list[int]:
-        return [g[0] for g in self.groups]
-
-    def row_ends(self) -> list[int]:
-        return [min(g[1], self.M) for g in self.groups]
-
-    def tile_counts(self) -> list[int]:
-        return [g[2] for g in self.groups]
+    def tile_counts(self) -> "list[int]":
+        return [tiles for _, _, tiles in self.groups]
 
 
 def _check_geometry(M, N, tile_bytes, block_m, block_n, group_m, max_groups) -> None:
@@ -114,18 +93,9 @@ def _check_geometry(M, N, tile_bytes, block_m, block_n, group_m, max_groups) -> 
         raise ValueError("max_groups must be positive")
 
 
-def build_tile_groups(
-    M: int,
-    N: int,
-    tile_bytes: int,
-    *,
-    target_group_tiles: int | None = None,
-    max_groups: int = 64,
-    block_m: int = DEFAULT_BLOCK_M,
-    block_n: int = DEFAULT_BLOCK_N,
-    group_m: int = DEFAULT_GROUP_M,
-    tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES,
-) -> list[TileGroup]:
+def build_tile_groups(M: int, N: int, tile_bytes: int, *, target_group_tiles: "int | None" = None, max_groups: int = 64,
+                      block_m: int = DEFAULT_BLOCK_M, block_n: int = DEFAULT_BLOCK_N, group_m: int = DEFAULT_GROUP_M,
+                      tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES) -> "list[TileGroup]":
     """Cut ``[0, M)`` into wave-aligned row bands of at least ``g_min`` tiles each.
 
     Walks the swizzle waves in order, closing a band as soon as it holds enough tiles.
@@ -159,26 +129,13 @@ def build_tile_groups(
 
     if len(bands) > max_groups:
         stride = _cdiv(len(bands), max_groups)
-        bands = [
-            (
-                bands[i][0],
-                min(bands[min(i + stride, len(bands)) - 1][1], M),
-                sum(b[2] for b in bands[i : i + stride]),
-            )
-            for i in range(0, len(bands), stride)
-        ]
+        runs = [bands[i:i + stride] for i in range(0, len(bands), stride)]
+        bands = [(run[0][0], min(run[-1][1], M), sum(tiles for _, _, tiles in run)) for run in runs]
     return bands
 
 
-def split_groups_at_row_boundaries(
-    M: int,
-    N: int,
-    groups: Sequence[TileGroup],
-    row_boundaries: Sequence[int],
-    *,
-    block_m: int = DEFAULT_BLOCK_M,
-    block_n: int = DEFAULT_BLOCK_N,
-) -> list[TileGroup]:
+def split_groups_at_row_boundaries(M: int, N: int, groups: "Sequence[TileGroup]", row_boundaries: "Sequence[int]", *,
+                                   block_m: int = DEFAULT_BLOCK_M, block_n: int = DEFAULT_BLOCK_N) -> "list[TileGroup]":
     """Cut every band at each interior boundary so no band straddles two row owners.
 
     Tile counts of the pieces are recomputed from their row extent
@@ -198,24 +155,15 @@ def split_groups_at_row_boundaries(
     return pieces
 
 
-def split_groups_at_row_shards(
-    M: int,
-    N: int,
-    groups: Sequence[TileGroup],
-    *,
-    num_shards: int,
-    block_m: int = DEFAULT_BLOCK_M,
-    block_n: int = DEFAULT_BLOCK_N,
-) -> list[TileGroup]:
+def split_groups_at_row_shards(M: int, N: int, groups: "Sequence[TileGroup]", *, num_shards: int,
+                               block_m: int = DEFAULT_BLOCK_M, block_n: int = DEFAULT_BLOCK_N) -> "list[TileGroup]":
     """Cut bands at the borders of ``num_shards`` equal row shards."""
     if num_shards <= 0:
         raise ValueError("num_shards must be positive")
-    if M % num_shards != 0:
+    if M % num_shards:
         raise ValueError(f"M={M} must be divisible by num_shards={num_shards}")
-    rows = M // num_shards
-    return split_groups_at_row_boundaries(
-        M, N, groups, [rows * s for s in range(1, num_shards)], block_m=block_m, block_n=block_n
-    )
+    borders = range(M // num_shards, M, M // num_shards)
+    return split_groups_at_row_boundaries(M, N, groups, borders, block_m=block_m, block_n=block_n)
 
 
 def swizzled_tile_rows(tile_rows: int, tile_cols: int, group_m: int) -> np.ndarray:
@@ -241,15 +189,8 @@ def swizzled_tile_cols(tile_rows: int, tile_cols: int, group_m: int) -> np.ndarr
     return (ids % per_band) // height
 
 
-def build_group_table(
-    M: int,
-    N: int,
-    groups: Sequence[TileGroup],
-    *,
-    block_m: int = DEFAULT_BLOCK_M,
-    block_n: int = DEFAULT_BLOCK_N,
-    group_m: int = DEFAULT_GROUP_M,
-) -> torch.Tensor:
+def build_group_table(M: int, N: int, groups: "Sequence[TileGroup]", *, block_m: int = DEFAULT_BLOCK_M,
+                      block_n: int = DEFAULT_BLOCK_N, group_m: int = DEFAULT_GROUP_M) -> torch.Tensor:
     """``int32[total_tiles]`` on the CPU: swizzled tile id -> group id.
 
     A tile belongs to the first group whose ``[row_start, row_end)`` contains the tile's
@@ -266,45 +207,17 @@ def build_group_table(
     return torch.from_numpy(table)
 
 
-def build_tile_group_plan(
-    M: int,
-    N: int,
-    tile_bytes: int,
-    *,
-    target_group_tiles: int | None = None,
-    max_groups: int = 64,
-    block_m: int = DEFAULT_BLOCK_M,
-    block_n: int = DEFAULT_BLOCK_N,
-    group_m: int = DEFAULT_GROUP_M,
-    tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES,
-    row_split_boundaries: Iterable[int] | None = (),
-) -> TileGroupPlan:
+def build_tile_group_plan(M: int, N: int, tile_bytes: int, *, target_group_tiles: "int | None" = None, max_groups: int = 64,
+                          block_m: int = DEFAULT_BLOCK_M, block_n: int = DEFAULT_BLOCK_N, group_m: int = DEFAULT_GROUP_M,
+                          tau_min_bytes: int = DEFAULT_TAU_MIN_BYTES,
+                          row_split_boundaries: "Iterable[int] | None" = ()) -> TileGroupPlan:
     """Groups (optionally cut at owner boundaries) plus their swizzle table, as one plan."""
-    groups = build_tile_groups(
-        M,
-        N,
-        tile_bytes,
-        target_group_tiles=target_group_tiles,
-        max_groups=max_groups,
-        block_m=block_m,
-        block_n=block_n,
-        group_m=group_m,
-        tau_min_bytes=tau_min_bytes,
-    )
+    tiling = dict(block_m=block_m, block_n=block_n)
+    sizing = dict(target_group_tiles=target_group_tiles, max_groups=max_groups, tau_min_bytes=tau_min_bytes)
+    groups = build_tile_groups(M, N, tile_bytes, group_m=group_m, **tiling, **sizing)
     cuts = list(row_split_boundaries or ())  # None: no boundaries, as the reference accepts (tile_group.py:269)
     if cuts:
-        groups = split_groups_at_row_boundaries(M, N, groups, cuts, block_m=block_m, block_n=block_n)
-    return TileGroupPlan(
-        M=M,
-        N=N,
-        tile_bytes=tile_bytes,
-        target_group_tiles=target_group_tiles,
-        max_groups=max_groups,
-        groups=groups,
-        group_table=build_group_table(M, N, groups, block_m=block_m, block_n=block_n, group_m=group_m),
-        block_m=block_m,
-        block_n=block_n,
-        group_m=group_m,
-        tau_min_bytes=tau_min_bytes,
-        p0_min_tiles=max(1, _cdiv(tau_min_bytes, tile_bytes)),
-    )
+        groups = split_groups_at_row_boundaries(M, N, groups, cuts, **tiling)
+    table = build_group_table(M, N, groups, group_m=group_m, **tiling)
+    return TileGroupPlan(M=M, N=N, tile_bytes=tile_bytes, groups=groups, group_table=table, group_m=group_m,
+                         p0_min_tiles=max(1, _cdiv(tau_min_bytes, tile_bytes)), **tiling, **sizing)
