@@ -141,3 +141,108 @@ def test_contract_errors(lib):
     finally:
         for c in ctxs:
             c.heap.cleanup()
+
+
+def test_ops_level_collectives_and_their_plans(lib):
+    """tileccl.ops.allgather / allreduce / reduce_scatter (reference ops.py:1083-1258): the same results
+    as the launchers underneath, plans that can be executed again, and validation that notices a tensor
+    the plan was not built for."""
+    import tileccl_amd as tileccl
+
+    world, block = 3, 2048
+    ctxs = contexts(world, 64 << 20)
+    try:
+        cpu = [seeded((block,), 50 + r) for r in range(world)]
+        srcs = [put(c, t) for c, t in zip(ctxs, cpu)]
+        outs = [c.zeros(world * block, dtype=torch.float16) for c in ctxs]
+        for r, c in enumerate(ctxs):
+            assert tileccl.ops.allgather(srcs[r], outs[r], ctx=c) is outs[r]
+        torch.cuda.synchronize()
+        for r, want in enumerate(oracle.allgather(cpu)):
+            assert torch.equal(bits(outs[r]).cpu(), bits(want))
+
+        wide = [seeded((world * block,), 60 + r) for r in range(world)]
+        ins = [put(c, t) for c, t in zip(ctxs, wide)]
+        shards = [c.zeros(block, dtype=torch.float16) for c in ctxs]
+        plans = [tileccl.ops.build_reduce_scatter_plan(ins[r], shards[r], ctx=c) for r, c in enumerate(ctxs)]
+        assert plans[0].to_dict()["block_size"] == block and plans[0].to_dict()["context"]["world_size"] == world
+        for _ in range(2):  # a plan is reusable
+            for r, plan in enumerate(plans):
+                plan.execute(ins[r], shards[r])
+        torch.cuda.synchronize()
+        for r, want in enumerate(oracle.reduce_scatter(wide, torch.float16)):
+            assert torch.equal(bits(shards[r]).cpu(), bits(want))
+        with pytest.raises(ValueError, match="reduce_scatter src shape no longer matches the plan"):
+            plans[0].execute(ins[0].reshape(world, block), shards[0])
+        with pytest.raises(ValueError, match="reduce_scatter src.numel must equal output.numel \\* world_size"):
+            tileccl.ops.reduce_scatter(srcs[0], shards[0], ctx=ctxs[0])
+        with pytest.raises(ValueError, match="implementation must be one of"):
+            tileccl.ops.reduce_scatter(ins[0], shards[0], ctx=ctxs[0], implementation="fast")
+
+        xs = [put(c, t) for c, t in zip(ctxs, wide)]
+        for r, c in enumerate(ctxs):
+            assert tileccl.ops.allreduce(xs[r], ctx=c) is xs[r]
+        torch.cuda.synchronize()
+        for r, want in enumerate(oracle.allreduce(wide)):
+            assert torch.equal(bits(xs[r]).cpu(), bits(want))
+        with pytest.raises(ValueError, match="allreduce currently supports only op='sum'"):
+            tileccl.ops.allreduce(xs[0], ctx=ctxs[0], op="max")
+        with pytest.raises(ValueError, match="must reside in the attached symmetric heap"):
+            tileccl.ops.allreduce(torch.zeros(block, dtype=torch.float16, device="cuda"), ctx=ctxs[0])
+        with pytest.raises(ValueError, match="allgather currently requires src to be contiguous"):
+            tileccl.ops.allgather(ins[0][::2], outs[0], ctx=ctxs[0])
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()
+
+
+def test_ops_level_gemm_plans_and_the_chained_op(lib):
+    """build_gemm_allgather_plan / build_gemm_reducescatter_plan / allgather_gemm_reducescatter
+    (reference ops.py:891-1080, 2315-2375) on the fused launches."""
+    import tileccl_amd as tileccl
+
+    world, M, N, K = 2, 512, 512, 128
+    ctxs = contexts(world, 128 << 20)
+    try:
+        Ns = N // world
+        A_cpu, B_cpu = seeded((M, K), 0), seeded((K, N), 1, scale=K**-0.5)
+        As = [put(c, A_cpu) for c in ctxs]
+        Bsh = [put(c, B_cpu[:, r * Ns:(r + 1) * Ns].contiguous()) for r, c in enumerate(ctxs)]
+        Cs = [c.zeros(M, N, dtype=torch.float16) for c in ctxs]
+        plans = [tileccl.ops.build_gemm_allgather_plan(As[r], Bsh[r], Cs[r], ctx=c) for r, c in enumerate(ctxs)]
+        assert plans[1].to_dict()["contract"]["shard_cols"] == Ns
+        for r, plan in enumerate(plans):
+            assert plan.execute(As[r], Bsh[r], Cs[r]) is Cs[r]
+        torch.cuda.synchronize()
+        assert torch.equal(bits(Cs[0]), bits(Cs[1]))
+        assert_gemm_close(Cs[0], A_cpu.float() @ B_cpu.float(), tight=0.004)
+        small = [c.zeros(256, N, dtype=torch.float16) for c in ctxs]  # on every rank: the slices stay in step
+        with pytest.raises(ValueError, match="Tensor contract no longer matches this GemmAllGatherPlan"):
+            plans[0].execute(As[0][:256], Bsh[0], small[0])
+
+        Bs = [put(c, B_cpu) for c in ctxs]
+        shard_out = [c.zeros(M, Ns, dtype=torch.float16) for c in ctxs]
+        rs = [tileccl.ops.build_gemm_reducescatter_plan(As[r], Bs[r], shard_out[r], ctx=c) for r, c in enumerate(ctxs)]
+        for _ in range(2):
+            for r, plan in enumerate(rs):
+                plan.execute(As[r], Bs[r], shard_out[r])
+        torch.cuda.synchronize()
+        full = world * (A_cpu.float() @ B_cpu.float())
+        for r in range(world):
+            assert_gemm_close(shard_out[r], full[:, r * Ns:(r + 1) * Ns], tight=0.008)
+
+        Ks = K // world
+        shards_cpu = [seeded((M, Ks), 30 + p) for p in range(world)]
+        shards = [put(c, s) for c, s in zip(ctxs, shards_cpu)]
+        outs = [c.zeros(M, N, dtype=torch.float16) for c in ctxs]
+        got = tileccl.ops.allgather_gemm_reducescatter(shards[1], Bs[1], outs[1], ctx=ctxs[1])
+        torch.cuda.synchronize()
+        assert got is outs[1]
+        assert_gemm_close(outs[1], oracle.gather_cols(shards_cpu).float() @ B_cpu.float(), tight=0.004)
+        with pytest.raises(ValueError, match=r"input_shard columns \(64\) \* world_size \(2\) must equal W rows \(192\)"):
+            tileccl.ops.allgather_gemm_reducescatter(shards[0], ctxs[0].zeros(192, N, dtype=torch.float16), outs[0], ctx=ctxs[0])
+        with pytest.raises(ValueError, match=r"output rows \(256\) must equal input_shard rows \(512\)"):
+            tileccl.ops.allgather_gemm_reducescatter(shards[0], Bs[0], small[0], ctx=ctxs[0])
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()

@@ -28,6 +28,23 @@ from tileccl_amd.patterns.contracts import PatternExecutionSpec, resolve_pattern
 __all__ = [
     "gemm_allgather",
     "gemm_reducescatter",
+    "allgather",
+    "allreduce",
+    "reduce_scatter",
+    "allgather_gemm_reducescatter",
+    "build_allgather_plan",
+    "build_allreduce_plan",
+    "build_reduce_scatter_plan",
+    "build_gemm_allgather_plan",
+    "build_gemm_reducescatter_plan",
+    "build_allgather_gemm_reducescatter_plan",
+    "AllGatherPlan",
+    "AllReducePlan",
+    "ReduceScatterPlan",
+    "GemmAllGatherPlan",
+    "GemmReduceScatterPlan",
+    "AllGatherGemmReduceScatterPlan",
+    "AllGatherGemmReduceScatterContract",
     "gemm_allscatter",
     "gemm_allscatter_sharded",
     "build_gemm_allscatter_plan",
@@ -37,6 +54,25 @@ __all__ = [
 ]
 
 from tileccl_amd.ops_collective import gemm_allgather, gemm_reducescatter  # noqa: E402  (re-exported)
+from tileccl_amd.ops_plans import (  # noqa: E402  (re-exported)
+    AllGatherGemmReduceScatterContract,
+    AllGatherGemmReduceScatterPlan,
+    AllGatherPlan,
+    AllReducePlan,
+    GemmAllGatherPlan,
+    GemmReduceScatterPlan,
+    ReduceScatterPlan,
+    allgather,
+    allgather_gemm_reducescatter,
+    allreduce,
+    build_allgather_gemm_reducescatter_plan,
+    build_allgather_plan,
+    build_allreduce_plan,
+    build_gemm_allgather_plan,
+    build_gemm_reducescatter_plan,
+    build_reduce_scatter_plan,
+    reduce_scatter,
+)
 
 PatternLike = str | type[Pattern] | Pattern | None
 LayoutKind = Literal["full", "shard"]
