@@ -159,7 +159,9 @@ def test_pattern_resolution_by_name_class_instance():
 def test_auto_select_reference_tree_and_measured_policy():
     """Each branch of the reference's decision tree (auto_select.py:128-188), by hand, at its
     default hardware (132 units, 300 GB/s -> bw_scale 1), and the policy used on MI355X."""
-    from tileccl_amd.patterns import auto_select as sel
+    import importlib
+
+    sel = importlib.import_module("tileccl_amd.patterns.auto_select")  # the package re-exports the function of that name
     from tileccl_amd.patterns.hip_patterns import BulkSyncPattern, TileGroupPattern, WGSpecializedPattern
 
     ref = lambda M, N, K, ws: sel.reference_choice(M, N, K, ws, 132, 300.0)  # noqa: E731

@@ -100,8 +100,12 @@ from tileccl_amd.patterns.hip_patterns import (  # noqa: E402
     WGSpecializedPattern,
 )
 
+from tileccl_amd.patterns.auto_select import auto_select, benchmark_all_patterns  # noqa: E402
+
 __all__ = [
     "Pattern",
+    "auto_select",
+    "benchmark_all_patterns",
     "BulkSyncPattern",
     "FusedSequentialPattern",
     "ProducerConsumerPattern",
