@@ -241,3 +241,21 @@ def test_b_operand_layouts():
         _launch._b_layout(torch.zeros(64, 256, dtype=torch.float16)[:, ::2])
     with pytest.raises(ValueError, match="2-D"):
         _launch._b_layout(torch.zeros(4, 4, 4))
+
+
+def test_context_and_pattern_helper_methods():
+    """TileCCLContext.auto_select_pattern / support_matrix (reference __init__.py:180-206) and
+    Pattern.require_device_remote_access_runtime (reference patterns/__init__.py:171-185)."""
+    import tileccl_amd
+    from tileccl_amd.patterns import Pattern
+    from tileccl_amd.patterns.hip_patterns import BulkSyncPattern, TileGroupPattern
+
+    ctx = tileccl_amd.TileCCLContext(rank=0, world_size=2, device="cuda:0", backend_name="hip", backend=None)
+    chosen = ctx.auto_select_pattern("gemm_allscatter", 4096, 8192, 1024)
+    assert type(chosen) is TileGroupPattern and chosen.ctx is ctx
+    one = tileccl_amd.TileCCLContext(rank=0, world_size=1, device="cuda:0", backend_name="hip", backend=None)
+    assert type(one.auto_select_pattern("gemm_allscatter", 4096, 8192, 1024)) is BulkSyncPattern
+    m = ctx.support_matrix().to_dict()
+    assert m["context"]["world_size"] == 2 and m["context"]["has_heap"] is False
+    with pytest.raises(RuntimeError):  # no heap attached: the guard needs one, as every pattern does
+        Pattern.require_device_remote_access_runtime(chosen, operation="gemm_allscatter")

@@ -144,3 +144,26 @@ def test_group_size_rule_prices_a_group_inside_a_launch_without_the_launch():
     slow = HardwareProfile(alpha_us=9.2, beta_us_per_byte=1e6 / 150e9, gemm_tflops_fp16=2500.0, gemm_efficiency=0.4,
                            min_comm_us=7.2, name="link")
     assert Calibration((), slow, 1000.0, 1).target_group_tiles(8192, 4096, 1024) >= 256
+
+
+def test_allreduce_cost_is_two_pipelines_of_the_shard_transfers():
+    """M = 1024 rows over 4 ranks, 128-tiles: a shard is 2 x 4 = 8 tiles, each half moves 3 shards = 24 tiles.
+    With alpha = 1 us, 1 GB/s... chosen so that a tile's transfer (32 KiB) and compute are round numbers."""
+    from tileccl_amd.v2.cost_model import HardwareProfile, TileCostModel
+
+    profile = HardwareProfile(alpha_us=1.0, beta_us_per_byte=1.0 / 32768, gemm_tflops_fp16=1.0, gemm_efficiency=1.0, name="toy")
+    model = TileCostModel(profile)
+    one = model.tile_cost(128, 128, 512, "float16")
+    assert one.comm_us == pytest.approx(2.0)  # 1 us + 32768 B at 32768 B/us
+    cost = model.allreduce_cost(1024, 512, 512, world_size=4)
+    assert set(cost) == {"reduce_scatter", "allgather", "total"}
+    for half in ("reduce_scatter", "allgather"):
+        assert len(cost[half].tile_costs) == 24
+        assert cost[half].sequential_us == pytest.approx(24 * one.sequential_us)
+        assert cost[half].pipelined_us == pytest.approx(one.sequential_us + 23 * one.overlapped_us)
+    total = cost["total"]
+    assert len(total.tile_costs) == 48
+    assert total.sequential_us == pytest.approx(48 * one.sequential_us)
+    assert total.pipelined_us == pytest.approx(2 * (one.sequential_us + 23 * one.overlapped_us))
+    assert total.overlap_ratio == pytest.approx(1.0 - total.pipelined_us / total.sequential_us)
+    assert total.bottleneck == cost["reduce_scatter"].bottleneck

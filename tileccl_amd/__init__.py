@@ -130,6 +130,18 @@ class TileCCLContext:
             t.zero_()
         return t
 
+    # -- pattern choice and support report (reference __init__.py:180-206) ---------------
+    def auto_select_pattern(self, op: str, M: int, N: int, K: int, *, hw_info: object | None = None):
+        """The pattern ``auto_select`` picks for this problem, bound to this context."""
+        from tileccl_amd.patterns.auto_select import auto_select
+
+        return auto_select(op, M=M, N=N, K=K, world_size=self.world_size, hw_info=hw_info, ctx=self)
+
+    def support_matrix(self):
+        from tileccl_amd.support import describe_runtime_support
+
+        return describe_runtime_support(self)
+
     # -- introspection ---------------------------------------------------------------
     def heap_metadata(self) -> dict[str, object]:
         return self.require_heap().metadata()

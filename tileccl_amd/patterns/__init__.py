@@ -92,6 +92,15 @@ class Pattern(abc.ABC):
         )
 
 
+def _require_device_remote_access_runtime(self, *, operation: str) -> None:
+    """The reference's guard against transports whose memory a device kernel cannot reach
+    (patterns/__init__.py:171-185).  Every heap of this build is a slice of one device arena,
+    reachable by plain loads and stores, so there is nothing to refuse; a heap is still required."""
+    self.ctx.require_heap()
+
+
+Pattern.require_device_remote_access_runtime = _require_device_remote_access_runtime
+
 from tileccl_amd.patterns.hip_patterns import (  # noqa: E402
     BulkSyncPattern,
     FusedSequentialPattern,

@@ -209,6 +209,28 @@ class TileCostModel:
                 best_size, best = edge, cost
         return best_size, best
 
+    def allreduce_cost(self, M: int, N: int, K: int, world_size: int, tile_size: int = 128,
+                       dtype: str = "float16") -> "dict[str, PipelineCost]":
+        """All-reduce of an ``M x N`` output priced as its two halves (reference
+        ``tileccl_v2/cost_model.py:381-432``): a reduce-scatter and an all-gather, each a pipeline of the
+        ``(world_size - 1)`` transfers of a rank's row shard, tile by tile; ``total`` adds the two
+        (no overlap between the halves is assumed)."""
+        shard_tiles = math.ceil((M // world_size) / tile_size) * math.ceil(N / tile_size)
+        halves = {
+            name: self.pipeline_cost(n_tiles=shard_tiles * (world_size - 1), tile_M=tile_size, tile_N=tile_size, tile_K=K, dtype=dtype)
+            for name in ("reduce_scatter", "allgather")
+        }
+        sequential = sum(h.sequential_us for h in halves.values())
+        pipelined = sum(h.pipelined_us for h in halves.values())
+        halves["total"] = PipelineCost(
+            tile_costs=[c for h in list(halves.values()) for c in h.tile_costs],
+            sequential_us=sequential,
+            pipelined_us=pipelined,
+            overlap_ratio=(1.0 - pipelined / sequential) if sequential > 0 else 0.0,
+            bottleneck=halves["reduce_scatter"].bottleneck,
+        )
+        return halves
+
     # -- TileGroup sizing ---------------------------------------------------
     def group_pipeline_us(
         self, n_groups: int, group_tiles: int, tile_M: int, tile_N: int, K: int, dtype: str, parallel_tiles: int
