@@ -301,7 +301,7 @@ int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* stag
  *             wait per tile (WGSpecializedPattern, wg_specialized.py:212-352).
  * variant S2: one launch; GEMM workgroups add to counter[group_table[tile]];
  *             communication workgroups wait per TileGroup and move copy_elems-sized
- *             tasks (reference README.md:66-84; contract in tileccl_v2/*.py).
+ *             tasks (reference README.md:66-84; contract in the tileccl_v2 modules).
  * With the 256 x 256 GEMM tile (gemm->macro_tile) S1 and S2 are still one launch, but a
  * workgroup fills its CU, so the communication is done by the GEMM workgroups themselves:
  * pushes leave from the epilogue, all-gather pulls run inside the K loop (S2) or after the
