@@ -304,8 +304,9 @@ int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* stag
  *             tasks (reference README.md:66-84; contract in the tileccl_v2 modules).
  * With the 256 x 256 GEMM tile (gemm->macro_tile) S1 and S2 are still one launch, but a
  * workgroup fills its CU, so the communication is done by the GEMM workgroups themselves:
- * pushes leave from the epilogue, all-gather pulls run inside the K loop (S2) or after the
- * workgroup's last tile (S1), reduce-scatter tiles are reduced right after they are
+ * pushes leave from the epilogue, all-gather pulls run inside the K loops (gated on the
+ * TileGroup counters in S2, on the per-tile locks in S1; what the K loops did not cover follows
+ * the workgroup's last tile), reduce-scatter tiles are reduced right after they are
  * published.  barrier[g] then advances by the grid size per launch, not by the task count.
  * Every device-side wait is bounded by sync->spin_limit_ns; an expired wait sets *sync->fault
  * and the kernel still runs to its end. */
@@ -319,9 +320,11 @@ int tccl_gemm_allscatter(const tccl_gemm_desc* gemm, const tccl_scatter_desc* sc
 /* ChainedAGGemmRSPattern.execute (patterns/chained_ag_gemm_rs.py:120-200): gather the ranks'
  * column shards of the input into gemm->A (M x K, K = world * k_shard, in this rank's slice),
  * output = gathered @ W (gemm->B), and store every output tile into every peer's output at
- * the same offset (scatter worker, :393-425).  The gather is one bulk launch ahead of the
- * GEMM; `variant` selects how the GEMM and the stores to the peers overlap (S0: GEMM kernel,
- * then a copy kernel; S1/S2: one launch, as tccl_gemm_allscatter). */
+ * the same offset (scatter worker, :393-425).  `variant` selects how the three stages overlap.
+ * S0: a gather launch, the GEMM kernel, then a copy kernel.  S1 / S2: one launch as
+ * tccl_gemm_allscatter, in which (256 x 256 tile, output of the input type, row-major B) the K
+ * loops read every rank's shard where it lies while gemm->A is filled in their background;
+ * otherwise the gather is a bulk launch of its own ahead of that launch. */
 int tccl_chained_ag_gemm_rs(const tccl_gemm_desc* gemm, const void* shard, int64_t ld_shard, int32_t k_shard,
                             const tccl_heap_view* heap, const tccl_sync_desc* sync,
                             const tccl_transport_desc* transport, int32_t variant, void* stream);
