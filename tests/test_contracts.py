@@ -259,3 +259,19 @@ def test_context_and_pattern_helper_methods():
     assert m["context"]["world_size"] == 2 and m["context"]["has_heap"] is False
     with pytest.raises(RuntimeError):  # no heap attached: the guard needs one, as every pattern does
         Pattern.require_device_remote_access_runtime(chosen, operation="gemm_allscatter")
+
+
+def test_import_smoke_as_the_reference_has_it():
+    """The reference's tests/test_import_smoke.py:10-18 on this package, plus its ``__all__``
+    (tileccl/__init__.py:539-552): every public name resolves."""
+    import importlib
+
+    tileccl = importlib.import_module("tileccl_amd")
+    assert isinstance(tileccl.__version__, str)
+    assert callable(tileccl.init) and callable(tileccl.init_local)
+    assert importlib.import_module("tileccl_amd.ops") is not None
+    reference_all = ["__version__", "init", "init_local", "get_rank", "get_world_size", "current_context",
+                     "describe_runtime_support", "TileCCLContext", "Tile", "SymmetricHeap", "patterns", "ops"]
+    for name in reference_all:
+        assert name in tileccl.__all__ and getattr(tileccl, name) is not None, name
+    assert tileccl.Tile is tileccl.SymmetricHeap  # the reference's placeholder alias (tileccl/__init__.py:514-522)

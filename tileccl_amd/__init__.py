@@ -319,6 +319,7 @@ __all__ = [
     "current_context",
     "describe_runtime_support",
     "TileCCLContext",
+    "Tile",
     "SymmetricHeap",
     "patterns",
     "ops",
