@@ -271,6 +271,30 @@ class Workload:
         lib = _lib.load()
         return lambda _variant: _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
 
+    def s0_host_sync(self):
+        """S0 as the reference issues it (patterns/bulk_sync.py:120-135): the GEMM kernel, a device-wide
+        synchronize on the host, then the exchange kernel.  All-gather workloads only."""
+        import ctypes as C
+
+        import torch
+
+        from tileccl_amd import _launch, _lib
+
+        if self.kind != "ag":
+            return None
+        gemm, op, lib = self.gemm_only(), self.op, _lib.load()
+        view = _launch.heap_view(op.heap.get_heap_bases(), op.rank, op.world_size)
+        transport = _launch.transport_desc(op.directions, op.transport.copy_elems, op.transport.reduce_elems, op.num_comm_wgs)
+
+        def run(_variant):
+            gemm(_variant)
+            torch.cuda.synchronize()
+            rc = lib.tccl_exchange_rows(_launch.ptr(op.out), self.M, self.N, int(op.out.stride(0)), op.out.element_size(),
+                                        C.byref(view), C.byref(transport), _launch.stream_ptr())
+            _lib.check(rc, "tccl_exchange_rows")
+
+        return run
+
     def library_gemm(self):
         """The same GEMM by torch.matmul (the vendor's GEMM library), for context: B row-major as the
         configurations hold it, and B k-major, the layout that library is fastest with.  16-bit inputs only."""
@@ -524,6 +548,13 @@ def main() -> int:
         line["library_gemm"] = library
     if "s0" in results and "s2" in results:
         line["s2_vs_s0_speedup"] = round(results["s0"]["event_ms_mean"] / results["s2"]["event_ms_mean"], 4)
+    if "s0" in results and getattr(w, "s0_host_sync", None) and w.s0_host_sync():
+        _, ms = time_variant(w.s0_host_sync(), "s0", args.steps, args.warmup)
+        line["s0_host_sync"] = {
+            "ms": round(ms, 5),
+            "note": "S0 with the reference's host-side device synchronize between the GEMM and the exchange kernel "
+                    "(variants_ms.s0 orders the two kernels by the stream alone)",
+        }
     if "s0" in results:
         phase_ms = results["s0"]["event_ms_mean"] - gemm_mean
         line["exchange_phase"] = {
