@@ -271,6 +271,40 @@ class Workload:
         lib = _lib.load()
         return lambda _variant: _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
 
+    def device_trace(self, variant, macro_tile):
+        """One traced launch of `variant` on an operation of its own (stamps cost about 1 us per launch, so
+        the timed operation carries none): per TileGroup, when its last tile was published and when the
+        transfers that depend on it were finished, in us from the launch's first stamp."""
+        import torch
+
+        from tileccl_amd.v2 import FusedGemmAllGather, FusedGemmReduceScatter
+        from tileccl_amd.v2.runtime import TimelineRecorder
+
+        common = dict(block_m=self.block_m, macro_tile=macro_tile, target_group_tiles=self.group_tiles, trace=True)
+        if self.kind == "ag":
+            ops = [FusedGemmAllGather(h, self.M, self.N, torch.float16, directions="both", **common) for h in self.heaps]
+            ops[1].out[self.M:].copy_(self.peer_cpu)
+        else:
+            ops = [FusedGemmReduceScatter(h, self.M, self.N, partial_dtype=self.op.partial.dtype, out_dtype=self.op.out.dtype,
+                                          own_rows_in_registers=True, **common) for h in self.heaps]
+            ops[1].partial.copy_(self.peer_cpu)
+        op = ops[0]
+        op.mark_peers_ready()
+        for _ in range(3):  # the last launch's stamps are the ones read
+            for t in (op.signals.trace_start_clock, op.signals.trace_ready_clock, op.signals.trace_done_clock):
+                t.zero_()
+            op(self.A, self.B, variant, scale_a=self.scales[0], scale_b=self.scales[1])
+        op.check_faults()
+        rec = TimelineRecorder(benchmark=self.describe(variant), path_name=variant,
+                               metadata={"workload": self.name, "tile_groups": op.plan.n_groups})
+        rec.record_signal_state(op.signals, op.plan, rank=0)
+        spans = {e.name: e for e in rec.events}
+        us = lambda name, end: round((spans[name].end_ms if end else spans[name].start_ms) * 1e3, 2) if name in spans else None  # noqa: E731
+        table = {"rows": [list(g[:2]) for g in op.plan.groups],
+                 "ready_us": [us(f"group {g} produce", True) for g in range(op.plan.n_groups)],
+                 "done_us": [us(f"group {g} transfer", True) for g in range(op.plan.n_groups)]}
+        return rec, table
+
     def s0_host_sync(self):
         """S0 as the reference issues it (patterns/bulk_sync.py:120-135): the GEMM kernel, a device-wide
         synchronize on the host, then the exchange kernel.  All-gather workloads only."""
@@ -445,6 +479,9 @@ def main() -> int:
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--macro-tile", type=int, default=0, choices=[0, 128, 256],
                     help="GEMM tile: 0 lets the library choose, 128 / 256 force a kernel")
+    ap.add_argument("--timeline", default=None, metavar="PATH",
+                    help="also run one traced launch of the reported variant and write its per-TileGroup timeline "
+                         "(tileccl.timeline.v1 JSON) to PATH; the bench line then carries `device_trace`")
     ap.add_argument("--group-tiles", default="default",
                     help="tiles per TileGroup: 'default' (the planner's rule), 'auto' (calibrate this machine and ask the "
                          "cost model), or a number")
@@ -548,6 +585,10 @@ def main() -> int:
         line["library_gemm"] = library
     if "s0" in results and "s2" in results:
         line["s2_vs_s0_speedup"] = round(results["s0"]["event_ms_mean"] / results["s2"]["event_ms_mean"], 4)
+    if args.timeline and getattr(w, "device_trace", None):
+        recorder, table = w.device_trace(args.variant, args.macro_tile)
+        recorder.write_json(args.timeline)
+        line["device_trace"] = table
     if "s0" in results and getattr(w, "s0_host_sync", None) and w.s0_host_sync():
         _, ms = time_variant(w.s0_host_sync(), "s0", args.steps, args.warmup)
         line["s0_host_sync"] = {
