@@ -102,11 +102,15 @@ template <>
 struct Mfma<_Float16> {
   typedef f16x8 Vec;
   static TCCL_D f32x16 run(Vec a, Vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  // 16 x 16 x 32: lane l holds 8 consecutive k (group l / 16) of row / column l % 16 and gets
+  // D[4 * (l / 16) + e][l % 16], e = 0..3.
+  static TCCL_D f32x4 run16(Vec a, Vec b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<__bf16> {
   typedef bf16x8 Vec;
   static TCCL_D f32x16 run(Vec a, Vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  static TCCL_D f32x4 run16(Vec a, Vec b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 };
 
 // fp32 -> output element, round to nearest even (what a cast of the accumulator does in

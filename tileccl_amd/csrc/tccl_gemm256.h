@@ -14,14 +14,22 @@
 // fetches:
 //   A stage: row-major, 128 B per row (64 k of a 16-bit type, 128 k of fp8); chunk kc of row r
 //            lives in slot kc ^ ((r >> 1) & 7).
-//   B stage: natural [k][n]; 16-bit: 512 B per k row, chunk c of row k in slot c ^ (4 * (k & 3));
-//            fp8: 256 B per k row, chunk c of row k in slot c ^ (2 * (k & 7)).
+//   B stage: natural [k][n]; 16-bit: 512 B per k row, chunk c of row k in slot
+//            c ^ (4 * (k & 3)) ^ (2 * ((k >> 3) & 1)); fp8: 256 B per k row, chunk c of row k in slot
+//            c ^ (2 * (k & 7)).
 // A operands are read with ds_read_b128.  B operands are read with the transposing LDS reads
 // of gfx950 (semantics measured on the device, 16 lanes at a time):
 //   ds_read_b64_tr_b16: lane i supplies 4 consecutive n of k row i/4 at column block i%4; lane j
-//                       receives 4 consecutive k of column j (two reads = the 8 k of 32x32x16);
+//                       receives 4 consecutive k of column j (two reads = the 8 k a lane holds of
+//                       a 16x16x32 operand);
 //   ds_read_b64_tr_b8:  lane i supplies 8 consecutive n of k row i/2 at column block i%2; lane j
 //                       receives 8 consecutive k of column j (four reads = the 32 k of 32x32x64).
+//
+// MFMA shape.  16-bit inputs use v_mfma_f32_16x16x32, not 32x32x16: with operands held in registers
+// and nothing else running, the matrix pipes of the whole part sustain 1.49 PFLOP/s of 32x32x16 on
+// N(0,1) fp16 data (2.3 PFLOP/s on zeros: the rate depends on the data, i.e. on power), 1.86 PFLOP/s of
+// 16x16x32.  The K loop of this kernel ran at the 32x32x16 figure; on 16x16x32 the GEMM alone is 7-11 %
+// faster.  fp8 inputs use v_mfma_scale_f32_32x32x64_f8f6f4.
 //
 // Pipeline: LDS holds two stages.  The loads of step kt+1 are issued, woven between the
 // first MFMAs of step kt, into the stage step kt-1 has left.  The step's one barrier
@@ -178,6 +186,8 @@ constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter wor
 // alone, two 16-byte units per lane and step, so that its bookkeeping runs once per 2 KiB and
 // only where it is covered.
 constexpr int kPullWaves = 4;                           // wavefronts of a workgroup that pull
+constexpr int kPullLaneBytes = 32;                      // per-lane pull state kept in LDS (see PullLane)
+constexpr int kPullStateBytes = kPullWaves * 64 * kPullLaneBytes;
 constexpr int kPullLoads = 2;                           // 16-byte units per lane and piece
 constexpr int kPieceUnits = 64 * kPullLoads;            // units per piece
 
@@ -255,17 +265,32 @@ struct Gemm256 {
   char* lds;   // stage 0 (also the epilogue's staging area)
   char* lds1;  // stage 1
   char* bgw;   // landing words of the background transfer's counter fetches
+  char* pls;   // per-lane state of the pulling wavefronts (kPullStateBytes of LDS; nullptr: nothing pulls)
   const int tid, lane, wave, wm, wn;
   // A per-lane value the optimiser must treat as new at this point (blocks hoisting of what is derived from it).
   static TCCL_D int fresh(int v) {
     asm volatile("" : "+v"(v));
     return v;
   }
+  // The lane's number, counted afresh (two instructions): what the per-step code of the background
+  // transfer derives from it is then formed where it is used instead of sitting in registers through
+  // the K loop.
+  // A wavefront-uniform sum the optimiser must take as a whole: split up, its loop-invariant part is added
+  // to the per-lane offsets ahead of the K loop, one register per combination.
+  static TCCL_D uint32_t whole(uint32_t v) {
+    asm("" : "+s"(v));
+    return v;
+  }
+  static TCCL_D int lane_now() { return fresh((int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
+
 
   TCCL_D Gemm256(const GemmArgs& args, int pull_args_offset, int push_args_offset, int reduce_args_offset, char* stage0,
-                 char* stage1, char* landing_words, int gather_args_offset = -1)
-      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), gather_offset(gather_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
-        wm((threadIdx.x >> 6) >> 2), wn((threadIdx.x >> 6) & 3) {}
+                 char* stage1, char* landing_words, int gather_args_offset = -1, char* pull_lane_state = nullptr)
+      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), gather_offset(gather_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), pls(pull_lane_state), tid(threadIdx.x), lane(threadIdx.x & 63),
+        // the wavefront's number is the same in all its lanes: held in a scalar register, and with it the LDS
+        // addresses its loads land at (kept per lane they cost eight registers and a readfirstlane per load)
+        wave(__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)), wm(__builtin_amdgcn_readfirstlane(threadIdx.x >> 8)),
+        wn(__builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3)) {}
 
   typedef __attribute__((address_space(3))) void LdsVoid;
   typedef const __attribute__((address_space(4))) PullArgs* PullPtr;
@@ -281,7 +306,10 @@ struct Gemm256 {
   //   B k rows 4*(4w+i) .. +3    (lane l: k row + l/16, slot l%16)            fp8 inputs
   struct Source {
     __amdgpu_buffer_rsrc_t a, b;
-    uint32_t off_a[4], off_b[4];
+    // Pieces 0 and 1 per lane; pieces 2 and 3 lie a fixed distance behind them (pair_a, pair_b), which is
+    // added where a load is issued: half the registers through the K loop.
+    uint32_t off_a[2], off_b[2];
+    uint32_t pair_a, pair_b;
     uint32_t step_a, step_b;
     // kGatherA: `a` is the window onto the shard that holds K steps [kt_base, kt_switch)
     int kt_base, kt_switch, row0;
@@ -322,7 +350,7 @@ struct Gemm256 {
     else
       s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(((int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col)) * kEsz), 0x00020000);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 2; ++i) {
       const int row = 8 * (4 * wave + i) + (lane >> 3);
       const int kc = (lane & 7) ^ ((row >> 1) & 7);
       int64_t lda = g.lda;
@@ -336,9 +364,18 @@ struct Gemm256 {
         s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
       } else {
         const int k = 2 * (4 * wave + i) + (lane >> 5);
-        const int c = (lane & 31) ^ (4 * (k & 3));
+        const int c = (lane & 31) ^ (4 * (k & 3)) ^ (2 * ((k >> 3) & 1));
         s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
       }
+    }
+    // Piece i + 2 covers rows (k rows) 16 (2 * kBRowsPerPiece) further on; the swizzle terms repeat with
+    // that period (rows: (row >> 1) & 7; k rows: k & 3 resp. k & 7), and bit 3 of k (16-bit B) only
+    // depends on the wave.
+    {
+      int64_t lda = g.lda;
+      if constexpr (kGatherA) lda = late_kernarg_ptr<GatherArgs>(gather_offset)->ld_shard;
+      s.pair_a = (uint32_t)(16 * lda * kEsz);
+      s.pair_b = kBKMajor ? (uint32_t)(16 * g.ldb * kEsz) : (uint32_t)(2 * kBRowsPerPiece * g.ldb * kEsz);
     }
     s.step_a = kStepK * kEsz;
     s.step_b = kBKMajor ? (uint32_t)(kStepK * kEsz) : (uint32_t)(kStepK * g.ldb * kEsz);
@@ -354,19 +391,19 @@ struct Gemm256 {
   TCCL_D void issue_a(char* stage, const Source& s, int kt, int i) const {
     const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);  // as in make_source
     const bool dead = kt * kStepK + kc * kChunkK >= g.K;
-    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + (kGatherA ? kt - s.kt_base : kt) * s.step_a;
+    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i & 1] + ((kGatherA ? kt - s.kt_base : kt) * s.step_a + (i >> 1) * s.pair_a);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + 8 * (4 * wave + i) * kARow256), 16, oa, 0, 0, 0);
   }
   TCCL_D void issue_b(char* stage, const Source& s, int kt, int i) const {
     if constexpr (kBKMajor) {
       const int kc = (lane & 7) ^ ((4 * (i & 1) + (lane >> 4)) & 7);
       const bool dead = kt * kStepK + kc * kChunkK >= g.K;
-      const uint32_t ob = dead ? 0xfffffff0u : s.off_b[i] + kt * s.step_b;
+      const uint32_t ob = dead ? 0xfffffff0u : s.off_b[i & 1] + whole(kt * s.step_b + (i >> 1) * s.pair_b);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + 8 * (4 * wave + i) * kARow256), 16, ob, 0, 0, 0);
       return;
     }
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage256 + (4 * wave + i) * 1024), 16,
-                                             s.off_b[i] + kt * s.step_b, 0, 0, 0);
+                                             s.off_b[i & 1] + whole(kt * s.step_b + (i >> 1) * s.pair_b), 0, 0, 0);
   }
   TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
     issue_a(stage, s, kt, i);
@@ -377,27 +414,40 @@ struct Gemm256 {
   struct Reader {
     uint32_t a_base;   // row of this lane in the A stage
     uint32_t a_swz;    // XOR term of the A slot
-    uint32_t b_base0;  // B address for column block bj = 0 (bj = 1 is b_base0 ^ 64), k row of kk = 0, q = 0
+    uint32_t b_base0;  // B address for the first column block, first k block (the others: load_b8 / load_b16)
   };
 
   TCCL_D Reader make_reader() const {
-    const int half = lane >> 5, l32 = lane & 31, i16 = lane & 15, grp = (lane >> 4) & 1;
-    const int t = i16 >> 2, cq = i16 & 3;
+    const int i16 = lane & 15;
     Reader r;
-    r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
-    r.a_swz = (uint32_t)((l32 >> 1) & 7);
-    if constexpr (kBKMajor) {
-      r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + l32) * kARow256);  // this lane's row of column block 0
-    } else if constexpr (kFp8) {
-      // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns of k row i/2
-      // (column block i%2) and lane j receives 8 consecutive k of column j.  Four reads
-      // (k + 0, 8, 16, 24) give the 32 consecutive k of v_mfma_f32_32x32x64_f8f6f4.
-      const int krow = i16 >> 1;
-      const int chunk = (wn * 4 + grp) ^ (2 * krow);
-      r.b_base0 = (uint32_t)(kAStage256 + (32 * half + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
+    if constexpr (!kFp8) {
+      // 16 x 16 x 32 operands: lane l reads row (column) l % 16 of a 16-row block, k group l / 16.
+      const int kg = lane >> 4, t = i16 >> 2, cq = i16 & 3;
+      r.a_base = (uint32_t)((wm * 128 + i16) * kARow256);
+      r.a_swz = (uint32_t)((i16 >> 1) & 7);
+      if constexpr (kBKMajor) {
+        r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + i16) * kARow256);  // this lane's row of column block 0
+      } else {
+        // ds_read_b64_tr_b16: within 16 lanes, lane i supplies 4 consecutive columns (4 * (i % 4) ..) of
+        // k row i / 4 and lane j receives those 4 k of column j.  Lane group kg covers k rows 8 * kg ..
+        // + 7 in two reads (k + 0, k + 4).
+        const int chunk = (wn * 8 + (cq >> 1)) ^ (4 * t) ^ (2 * (kg & 1));
+        r.b_base0 = (uint32_t)(kAStage256 + (8 * kg + t) * kBPitch + chunk * 16 + (cq & 1) * 8);
+      }
     } else {
-      const int chunk = (wn * 8 + grp * 2 + (cq >> 1)) ^ (4 * t);
-      r.b_base0 = (uint32_t)(kAStage256 + (8 * half + t) * kBPitch + chunk * 16 + (cq & 1) * 8);
+      const int half = lane >> 5, l32 = lane & 31, grp = (lane >> 4) & 1;
+      r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
+      r.a_swz = (uint32_t)((l32 >> 1) & 7);
+      if constexpr (kBKMajor) {
+        r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + l32) * kARow256);  // this lane's row of column block 0
+      } else {
+        // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns of k row i/2
+        // (column block i%2) and lane j receives 8 consecutive k of column j.  Four reads
+        // (k + 0, 8, 16, 24) give the 32 consecutive k of v_mfma_f32_32x32x64_f8f6f4.
+        const int krow = i16 >> 1;
+        const int chunk = (wn * 4 + grp) ^ (2 * krow);
+        r.b_base0 = (uint32_t)(kAStage256 + (32 * half + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
+      }
     }
     return r;
   }
@@ -444,30 +494,28 @@ struct Gemm256 {
     return __builtin_bit_cast(Vec, v);
   }
 
-  // 16-bit operands of k-block kk (16 k): the A rows of slab bi; the B columns of both blocks.
-  TCCL_D Vec load_a16(const char* stage, const Reader& r, int kk, int bi) const {
-    const int half = lane >> 5;
-    return *(const Vec*)(stage + r.a_base + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4) + bi * 32 * kARow256);
+  // 16-bit operands of k-block kh (32 k): the A rows of the 16-row block rb; the B columns of the
+  // wave's four 16-column blocks.
+  TCCL_D Vec load_a16(const char* stage, const Reader& r, int kh, int rb) const {
+    const int kg = lane >> 4;
+    return *(const Vec*)(stage + r.a_base + ((((uint32_t)(4 * kh + kg)) ^ r.a_swz) << 4) + rb * 16 * kARow256);
   }
-  TCCL_D void load_b16(const char* stage, const Reader& r, int kk, Vec (&fb)[2]) const {
+  TCCL_D Vec load_b16(const char* stage, const Reader& r, int kh, int cb) const {
     if constexpr (kBKMajor) {
-      const int half = lane >> 5;
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-        fb[b] = *(const Vec*)(stage + r.b_base0 + ((((uint32_t)(2 * kk + half)) ^ r.a_swz) << 4) + b * 32 * kARow256);
-      return;
+      const int kg = lane >> 4;
+      return *(const Vec*)(stage + r.b_base0 + ((((uint32_t)(4 * kh + kg)) ^ r.a_swz) << 4) + cb * 16 * kARow256);
     }
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const char* pb = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 64u)) + 16 * kk * kBPitch;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)pb);
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch));
-      const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      fb[b] = __builtin_bit_cast(Vec, both);
-    }
+    // column block cb: two chunks further on per block; the XOR commutes with the swizzle terms (they touch
+    // the chunk index only through XOR as well)
+    const char* pb = stage + (r.b_base0 ^ (uint32_t)(32 * cb)) + 32 * kh * kBPitch;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)pb);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch));
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(Vec, both);
   }
 
   // ---- background transfer -----------------------------------------------------------------------
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   struct PullState {
     int next_slot, next_lp;  // next piece of this wavefront: block slot, piece inside the block
     int stride;              // wavefronts in the grid
@@ -481,8 +529,12 @@ struct Gemm256 {
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
-    int pend_mask;           // bit per slot (K step parity): a piece was requested into it and is not yet stored
-    u32x4 piece[2][kPullLoads];  // the pieces themselves (slots are always named statically)
+    int pend_mask;           // non-zero: a piece was requested and is not yet stored
+    u32x4 seen_pos;          // pull_peek_*(): the lane's LDS state, held for the item between request and use
+    u32x2 seen_pend;
+    // The piece itself.  One set of registers: a piece is stored (pull_retire) before the next one is
+    // requested, in every path; a second set costs the fused kernels registers they do not have.
+    u32x4 piece[1][kPullLoads];
     int probe_off;           // this wavefront's counter landing words
     // The counter word, read out of the landing words right behind a K step's barrier: read
     // there, it is older than every operand fetch that follows, so using it never waits for those.
@@ -495,9 +547,6 @@ struct Gemm256 {
     uint32_t upr, pitch, units;
     int pieces, slots, n_groups;
     uint32_t adv_row, adv_col;   // what `stride` pieces add to (row, col)
-    uint32_t row[kPullLoads], col[kPullLoads];  // per lane: row / unit-in-row of this lane's units of piece next_lp
-    uint32_t pend_off[2][kPullLoads];  // per lane: byte offsets of the pending piece's units inside the block;
-                                       // kNoUnit: the unit does not exist (a block's last piece may be short)
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -529,11 +578,9 @@ struct Gemm256 {
     st.pend_mask = 0;
     st.probe_val = 0;
 #pragma unroll
-    for (int j = 0; j < kPullLoads; ++j) {
-      st.piece[0][j] = st.piece[1][j] = u32x4{0, 0, 0, 0};
-      st.row[j] = st.col[j] = 0;
-      st.pend_off[0][j] = st.pend_off[1][j] = 0;
-    }
+    for (int j = 0; j < kPullLoads; ++j) st.piece[0][j] = u32x4{0, 0, 0, 0};
+    st.seen_pos = u32x4{0, 0, 0, 0};
+    st.seen_pend = u32x2{0, 0};
     st.active = pull_offset >= 0 && a->mode != kBgNone && w < kPullWaves;
     st.primed = false;
     st.upr = st.pitch = st.units = 0;
@@ -555,26 +602,50 @@ struct Gemm256 {
     return st;
   }
 
-  // (row, col) of this lane's unit of piece next_lp, by division: at the start and when a block is finished.
+  // What a pulling lane carries from K step to K step besides the piece itself lives in LDS, not in
+  // registers (the fused kernels have none to spare, and a register spilled to scratch memory comes back
+  // through the same queue as the operand loads: a reload inside the K loop waits for all of them).
+  //   pos  = { row[0], row[1], col[0], col[1] }: row / unit-in-row of this lane's units of piece next_lp
+  //   pend = { off[0], off[1] }: byte offsets of the pending piece's units inside the block; kNoUnit: the
+  //          unit does not exist (a block's last piece may be short)
+  static_assert(kPullLoads == 2, "PullLane holds two units per lane");
+  TCCL_D char* pull_lane() const { return pls + (wave * 64 + lane_now()) * kPullLaneBytes; }  // wave < kPullWaves
+  TCCL_D u32x4 pull_pos() const { return *(const u32x4*)pull_lane(); }
+  TCCL_D void pull_set_pos(u32x4 pos) const { *(u32x4*)pull_lane() = pos; }
+  TCCL_D u32x2 pull_pend() const { return *(const u32x2*)(pull_lane() + 16); }
+  TCCL_D void pull_set_pend(u32x2 pend) const { *(u32x2*)(pull_lane() + 16) = pend; }
+  TCCL_D void pull_peek_pend(PullState& st) const {
+    if constexpr (kWithReduce) return;
+    if (st.active) st.seen_pend = pull_pend();
+  }
+  TCCL_D void pull_peek_pos(PullState& st) const {
+    if constexpr (kWithReduce) return;
+    if (st.active) st.seen_pos = pull_pos();
+  }
+
+  // (row, col) of this lane's units of piece next_lp, by division: at the start and when a block is finished.
   TCCL_D void pull_locate(PullState& st) const {
+    u32x4 pos;
 #pragma unroll
     for (int j = 0; j < kPullLoads; ++j) {
-      const uint32_t u = (uint32_t)st.next_lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane);
-      st.row[j] = u / st.upr;
-      st.col[j] = u - st.row[j] * st.upr;
+      const uint32_t u = (uint32_t)st.next_lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane_now());
+      pos[j] = u / st.upr;
+      pos[2 + j] = u - pos[j] * st.upr;
     }
+    pull_set_pos(pos);
   }
   // The same after next_lp += stride.
-  TCCL_D void pull_advance(PullState& st) const {
+  TCCL_D void pull_advance(PullState& st, u32x4 pos) const {
 #pragma unroll
     for (int j = 0; j < kPullLoads; ++j) {
-      st.row[j] += st.adv_row;
-      st.col[j] += st.adv_col;
-      if (st.col[j] >= st.upr) {
-        st.col[j] -= st.upr;
-        ++st.row[j];
+      pos[j] += st.adv_row;
+      pos[2 + j] += st.adv_col;
+      if (pos[2 + j] >= st.upr) {
+        pos[2 + j] -= st.upr;
+        ++pos[j];
       }
     }
+    pull_set_pos(pos);
   }
 
   // Fetch the first counters in the first tile's prologue, so that the first K step can
@@ -675,15 +746,16 @@ struct Gemm256 {
   // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.  The
   // piece belongs to the selected block: pull_issue() stores what is pending before it selects
   // another one.
-  TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int slot) const {
+  template <bool kPeeked = false>
+  TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int) const {
     if constexpr (kWithReduce) return false;
+    constexpr int slot = 0;
     if (!(st.pend_mask & (1 << slot))) return false;
     const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
+    const u32x2 pend = kPeeked ? st.seen_pend : pull_pend();
 #pragma unroll
-    for (int j = 0; j < kPullLoads; ++j) {
-      const uint32_t off = st.pend_off[slot][j];
-      if (off != kNoUnit) st16<kStreaming>(dst, off, st.piece[slot][j]);
-    }
+    for (int j = 0; j < kPullLoads; ++j)
+      if (pend[j] != kNoUnit) st16<kStreaming>(dst, pend[j], st.piece[slot][j]);
     st.pend_mask &= ~(1 << slot);
     return true;
   }
@@ -706,9 +778,10 @@ struct Gemm256 {
   // 2 gidx + 1; lanes beyond the grid look at a tile that exists (a duplicate).
   TCCL_D uint32_t probe_offset(PullPtr a, int gidx) const {
     if (!a->tile_mode) return (uint32_t)gidx * 4u;
-    int tm = 2 * gidx + (lane >> 5);
+    const int ln = lane_now();
+    int tm = 2 * gidx + (ln >> 5);
     if (tm >= g.tile_rows) tm = g.tile_rows - 1;
-    int tn = lane & 31;
+    int tn = ln & 31;
     if (tn >= g.tile_cols) tn = 0;
     const int sh = a->group_m_shift;
     const int first_m = (tm >> sh) << sh;
@@ -728,13 +801,15 @@ struct Gemm256 {
   TCCL_D void pull_collect(PullState& st, PullPtr a, const char* landing, int slot) const {
     if constexpr (kWithReduce) return;
     if (!st.active) return;
-    st.probe_val = *(const int32_t*)(bgw + st.probe_off + 4 * lane);  // lane l's word landed at 4 l
+    st.probe_val = *(const int32_t*)(bgw + st.probe_off + 4 * lane_now());  // lane l's word landed at 4 l
   }
   // Once per K step: learn about readiness, request the next piece into slot `slot` (its
   // previous piece was stored during the step before).  All control flow here is
   // wavefront-uniform.  Returns whether a piece was requested.
-  TCCL_D bool pull_issue(PullState& st, PullPtr a, char* landing, int slot) const {
+  template <bool kPeeked = false>
+  TCCL_D bool pull_issue(PullState& st, PullPtr a, char* landing, int) const {
     if constexpr (kWithReduce) return false;
+    constexpr int slot = 0;
     if (!st.active) return false;
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
@@ -748,7 +823,7 @@ struct Gemm256 {
     }
     if (st.next_slot >= st.slots) return false;
     if (st.next_slot != st.slot) {
-      pull_retire(st, a, landing, slot ^ 1);  // the piece of the step before belongs to the block being left
+      pull_retire(st, a, landing, slot);  // a piece still pending belongs to the block being left
       pull_select(st, a, st.next_slot);
       pull_probe(st, a, landing);
       return false;
@@ -758,22 +833,26 @@ struct Gemm256 {
     const uint32_t last = first + (uint32_t)(kPieceUnits - 1);
     if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
       const __amdgpu_buffer_rsrc_t src = window(st.src_base);
+      const u32x4 pos = kPeeked ? st.seen_pos : pull_pos();
+      u32x2 pend;
+      const int ln = lane_now();
 #pragma unroll
       for (int j = 0; j < kPullLoads; ++j) {
-        const bool valid = first + (uint32_t)(64 * j + lane) < st.units;
-        const uint32_t off = valid ? st.row[j] * st.pitch + st.col[j] * 16u : 0u;  // idle lanes touch the block's first unit
+        const bool valid = first + (uint32_t)(64 * j + ln) < st.units;
+        const uint32_t off = valid ? pos[j] * st.pitch + pos[2 + j] * 16u : 0u;  // idle lanes touch the block's first unit
         uint32_t from = off;
-        if constexpr (kGatherA) from = valid ? st.row[j] * a->src_pitch + st.col[j] * 16u : 0u;
+        if constexpr (kGatherA) from = valid ? pos[j] * a->src_pitch + pos[2 + j] * 16u : 0u;
         st.piece[slot][j] = ld16<kCoherent>(src, from);
-        st.pend_off[slot][j] = valid ? off : kNoUnit;
+        pend[j] = valid ? off : kNoUnit;
       }
+      pull_set_pend(pend);
       st.pend_mask |= 1 << slot;
       st.next_lp += st.stride;
       if (st.next_lp >= st.pieces) {  // block finished: rare, may divide
         pull_normalise(st, a);
         pull_locate(st);
       } else {
-        pull_advance(st);
+        pull_advance(st, pos);
       }
       return true;
     }
@@ -827,7 +906,6 @@ struct Gemm256 {
   TCCL_D bool pull_drain(PullState& st, PullPtr a, const char* landing) const {
     wait_vmem();
     pull_retire(st, a, landing, 0);
-    pull_retire(st, a, landing, 1);
     st.probe_group = -1;
     const int64_t deadline = now_ticks() + a->spin_ticks;
     bool ok = true;
@@ -881,7 +959,7 @@ struct Gemm256 {
 
   // 16-bit operand registers; they live across K steps.
   struct Frags {
-    Vec ring[4], fbr[2][2];
+    Vec ring[4], fb[4];
   };
 
   // fp8 operand registers; they live across K steps.
@@ -928,32 +1006,33 @@ struct Gemm256 {
     pull_retire(pull, pa(), bgw, parity);  // the piece this step requested: it arrived before the barrier
   }
 
-  // One K step of the 16-bit path: sixteen items (k-block kk, A slab bi) of two MFMAs each,
-  // read from `cur` while the next step's operands stream into `nxt`.
+  // One K step of the 16-bit path (v_mfma_f32_16x16x32): eight items of eight MFMAs each, read from `cur`
+  // while the next step's operands stream into `nxt`.  Item d covers k block kh = d / 4 (32 k) and the
+  // 16-row blocks 2 * (d % 4), + 1 of the wave tile, against all four 16-column blocks.
   //
-  // The operands of item i + 2 are fetched before the MFMAs of item i are issued, so an LDS
-  // read has two items (~130 clocks of matrix work, more with the SIMD's other wave) to come
-  // back; A rotates through four register sets, B through two, and the scheduling barriers pin
-  // this order (left alone, the compiler hoists every read of the step and spills).
+  // A operands (two per item) are fetched one item ahead through four register sets.  B operands
+  // (four per k block) have ONE register set: the last item of a k block runs column block by
+  // column block, and as soon as a column block's two MFMAs are issued its registers take the next k
+  // block's operand, which is first needed six MFMAs later (the first item of a k block runs in the
+  // same order).  A second set would cost 16 registers, which the fused kernels do not have.
+  // The scheduling barriers pin this order (left alone, the compiler hoists every read of the step and
+  // spills).
   //
-  // The step's one barrier sits before item 14, not at the end.  There this wave has issued
+  // The step's one barrier sits before the last item, not at the end.  There this wave has issued
   // (and, after the lgkmcnt wait, finished) its last read of `cur`, and its loads into `nxt`,
-  // issued during items 0..7, have landed; behind the barrier items 14 and 15 already fetch
+  // issued during items 0..3, have landed; behind the barrier the last item already fetches
   // the next step's first operands from `nxt`, so the matrix pipe does not drain while the
-  // first LDS reads of a step are in flight.  Measured against a barrier at the end of the
-  // step (4096^3 fp16): 128.4 us instead of 133.6.
+  // first LDS reads of a step are in flight.
   //
-  // The loads go out one per item over items 0..7.  Issuing a load holds the wave for as long
-  // as the address unit takes to accept it (about 16 clocks per KiB instruction, four times
-  // that when the four SIMDs' waves issue in the same item), and nothing else of the wave
-  // issues meanwhile; later or denser placements measured slower.
+  // Issuing a global load holds the wave for as long as the address unit takes to accept it (about 16
+  // clocks per KiB instruction, four times that when the four SIMDs' waves issue in the same item),
+  // and nothing else of the wave issues meanwhile; they go out two per item over items 0..3.
   TCCL_D void k_step16(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                        Frags& f, PullState& pull, int parity) const {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int kk = i >> 2, bi = i & 3;
-      const int j = (i + 2) & 15;
-      if (i == 14) {
+    for (int d = 0; d < 8; ++d) {
+      const int rp = d & 3;
+      if (d == 7) {
         // This wave's loads (and background fetch) have landed, its reads of `cur` are done.
         // The barrier is the bare instruction: __syncthreads() carries a workgroup-scope
         // release fence.  The empty asm keeps the compiler from moving LDS accesses across it.
@@ -962,31 +1041,60 @@ struct Gemm256 {
         asm volatile("" ::: "memory");
         pull_collect(pull, pa(), bgw, parity);
       }
-      const char* from = i + 2 < 16 ? cur : nxt;
-      if ((j & 3) == 0) load_b16(from, rd, j >> 2, f.fbr[(j >> 2) & 1]);
-      f.ring[(i + 2) & 3] = load_a16(from, rd, j >> 2, j & 3);
-      // One load per item over items 0..7 (A pieces on even items, B pieces on odd ones): 0.3-0.6 %
-      // ahead of issuing them as pairs on the even items.
-      if (i < 8) {
-        if ((i & 1) == 0)
-          issue_a(nxt, src, kt_load, i >> 1);
-        else
-          issue_b(nxt, src, kt_load, i >> 1);
+      const int dn = (d + 1) & 7;
+      const char* from = d + 1 < 8 ? cur : nxt;
+      f.ring[2 * (dn & 1)] = load_a16(from, rd, dn >> 2, 2 * (dn & 3));
+      f.ring[2 * (dn & 1) + 1] = load_a16(from, rd, dn >> 2, 2 * (dn & 3) + 1);
+      if (d < 4) {
+        issue_a(nxt, src, kt_load, d);
+        issue_b(nxt, src, kt_load, d);
       }
-      // The piece requested at the start of the step before (it arrived before that step's
-      // barrier) is stored here, away from the cluster of loads at a step's start: 0.4-1.8 %
-      // on the all-gather at 4096x4096x1024 against storing it at the end of its own step,
-      // 1.6 % against storing it right behind the barrier.
-      if (i == 9) pull_retire(pull, pa(), bgw, parity ^ 1);
+      // The pulling lanes' state comes out of LDS an item before it is used: asked for where it is
+      // used, the wait for it would also hold back this wave's MFMAs.
+      if (d == 1) pull_peek_pend(pull);
+      // The piece requested during the step before (it arrived before that step's barrier) is
+      // stored ahead of the next request, so that one set of piece registers serves both.
+      if (d == 2) {
+        pull_retire<true>(pull, pa(), bgw, parity ^ 1);
+        pull_peek_pos(pull);
+      }
       // The next piece is requested behind the step's last operand loads, not ahead of them:
       // loads complete in issue order, so a request that has to go out to the peer's memory
-      // would hold back every operand load issued after it (2.4 % on the same workload
-      // against requesting it at the step's start).
-      if (i == 7) pull_issue(pull, pa(), bgw, parity);
-      acc[bi][0] = Mfma<InT>::run(f.fbr[kk & 1][0], f.ring[i & 3], acc[bi][0]);
-      acc[bi][1] = Mfma<InT>::run(f.fbr[kk & 1][1], f.ring[i & 3], acc[bi][1]);
+      // would hold back every operand load issued after it.
+      if (d == 3) pull_issue<true>(pull, pa(), bgw, parity);
+      // acc[rb / 2][cb / 2] holds a 32 x 32 patch as four 16 x 16 blocks: registers 4 * q .. 4 * q + 3 are
+      // block q = 2 * (rb % 2) + cb % 2 (acc_spot() is the lane's place in it).
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int rb = 2 * rp + r;
+          f32x16& patch = acc[rb >> 1][cb >> 1];
+          const int q = 2 * (rb & 1) + (cb & 1);
+          f32x4 blk = {patch[4 * q], patch[4 * q + 1], patch[4 * q + 2], patch[4 * q + 3]};
+          blk = Mfma<InT>::run16(f.fb[cb], f.ring[2 * (d & 1) + r], blk);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) patch[4 * q + e] = blk[e];
+        }
+        if (rp == 3) {
+          __builtin_amdgcn_sched_barrier(0);
+          f.fb[cb] = load_b16(from, rd, dn >> 2, cb);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
+  }
+
+  // Where registers 4 * q .. 4 * q + 3 of acc[bi][bj] sit in the 32-row slab bi of the wave tile: row inside
+  // the slab, first of four consecutive columns inside the wave's 64.  fp8 (32 x 32 x 64 MFMA): lane l holds
+  // row l % 32, columns 8 * q + 4 * (l / 32) ..; 16-bit inputs (16 x 16 x 32 MFMA): block q of the patch,
+  // row l % 16 of it, columns 4 * (l / 16) .. .
+  struct Spot {
+    int row, col;
+  };
+  static TCCL_D Spot acc_spot(int ln, int bj, int q) {
+    if constexpr (kFp8) return Spot{ln & 31, bj * 32 + 8 * q + 4 * (ln >> 5)};
+    return Spot{16 * (q >> 1) + (ln & 15), bj * 32 + 16 * (q & 1) + 4 * (ln >> 4)};
   }
 
   // Stores the tile and, when a push is asked for, sends it to the peers from the same LDS staging.
@@ -1001,7 +1109,6 @@ struct Gemm256 {
     // invariant across tiles, gets hoisted out of the tile loop and occupies registers all
     // through the K loop.
     const int ln = fresh(lane);
-    const int half = ln >> 5, l32 = ln & 31;
     OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
     const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
     // Fields are read through the argument block itself: a local copy would sit in scalar
@@ -1019,13 +1126,13 @@ struct Gemm256 {
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n_local = bj * 32 + 8 * q + 4 * half;
+          const Spot at = acc_spot(ln, bj, q);
           OutT v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[bi][bj][4 * q + e] * g.alpha);
-          const int byte = n_local * kEsz;
-          const int chunk = (byte >> 4) ^ (l32 & 7);
-          char* p = win + l32 * kRowBytes + chunk * 16 + (byte & 15);
+          const int byte = at.col * kEsz;
+          const int chunk = (byte >> 4) ^ (at.row & 7);
+          char* p = win + at.row * kRowBytes + chunk * 16 + (byte & 15);
           if constexpr (kEsz == 2) {
             uint2 u;
             __builtin_memcpy(&u, v, 8);
@@ -1089,7 +1196,6 @@ struct Gemm256 {
     constexpr int kRounds = (32 * kChunks) / 64;
     char* win = lds + wave * (32 * 64 * 4);
     const int ln = fresh(lane);  // as in epilogue(): keeps the offsets below out of the K loop's registers
-    const int half = ln >> 5, l32 = ln & 31;
     const int world = ra->world, rank = ra->rank;
     const int64_t my_base = ra->heap_bases[rank];
     const int64_t tile_off = ((int64_t)row0 * g.ldc + col0) * kEsz;
@@ -1109,13 +1215,13 @@ struct Gemm256 {
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n_local = bj * 32 + 8 * q + 4 * half;
+          const Spot at = acc_spot(ln, bj, q);
           OutT v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[bi][bj][4 * q + e] * g.alpha);
-          const int byte = n_local * kEsz;
-          const int chunk = (byte >> 4) ^ (l32 & 7);
-          char* p = win + l32 * kRowBytes + chunk * 16 + (byte & 15);
+          const int byte = at.col * kEsz;
+          const int chunk = (byte >> 4) ^ (at.row & 7);
+          char* p = win + at.row * kRowBytes + chunk * 16 + (byte & 15);
           if constexpr (kEsz == 2) {
             uint2 u;
             __builtin_memcpy(&u, v, 8);
@@ -1234,7 +1340,8 @@ struct Gemm256 {
       }
     } else {
       Frags f;
-      load_b16(lds, rd, 0, f.fbr[0]);
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) f.fb[cb] = load_b16(lds, rd, 0, cb);
       f.ring[0] = load_a16(lds, rd, 0, 0);
       f.ring[1] = load_a16(lds, rd, 0, 1);
       for (int kt = 0; kt < ksteps; kt += 2) {
