@@ -275,3 +275,25 @@ def test_import_smoke_as_the_reference_has_it():
     for name in reference_all:
         assert name in tileccl.__all__ and getattr(tileccl, name) is not None, name
     assert tileccl.Tile is tileccl.SymmetricHeap  # the reference's placeholder alias (tileccl/__init__.py:514-522)
+
+
+def test_spill_check_reads_an_assembly_listing():
+    """tileccl_amd.csrc.check_spills counts scratch-memory instructions between a kernel's first and last MFMA."""
+    from tileccl_amd.csrc.check_spills import kernels
+
+    name = "_ZN4tccl15fused256_kernelIDF16_DF16_Lb0ELb0ELb0EEEvNS_12Fused256ArgsE"
+    asm = "\n".join([
+        f"{name}:                         ; @{name}",
+        "\tscratch_store_dword off, v2, off offset:8 ; 4-byte Folded Spill",
+        "\tv_mfma_f32_16x16x32_f16 v[0:3], v[4:7], v[8:11], v[0:3]",
+        "\tscratch_load_dword v178, off, off ; 4-byte Folded Reload",
+        "\tds_read_b128 v[4:7], v9",
+        "\tv_mfma_f32_16x16x32_f16 v[0:3], v[4:7], v[8:11], v[0:3]",
+        "\tscratch_load_dword v2, off, off offset:8 ; 4-byte Folded Reload",
+        "\ts_endpgm",
+        ".Lfunc_end0:",
+        "  - .name:           " + name,
+        "    .sgpr_count:     104",
+        "    .vgpr_count:     256",
+    ]) + "\n"
+    assert list(kernels(asm)) == [(name, 256, 1, 3)]
