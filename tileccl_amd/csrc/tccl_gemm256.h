@@ -16,20 +16,22 @@
 //            lives in slot kc ^ ((r >> 1) & 7).
 //   B stage: natural [k][n]; 16-bit: 512 B per k row, chunk c of row k in slot
 //            c ^ (4 * (k & 3)) ^ (2 * ((k >> 3) & 1)); fp8: 256 B per k row, chunk c of row k in slot
-//            c ^ (2 * (k & 7)).
+//            c ^ (2 * (k & 7)) ^ ((k >> 5) & 1).
 // A operands are read with ds_read_b128.  B operands are read with the transposing LDS reads
 // of gfx950 (semantics measured on the device, 16 lanes at a time):
 //   ds_read_b64_tr_b16: lane i supplies 4 consecutive n of k row i/4 at column block i%4; lane j
 //                       receives 4 consecutive k of column j (two reads = the 8 k a lane holds of
 //                       a 16x16x32 operand);
 //   ds_read_b64_tr_b8:  lane i supplies 8 consecutive n of k row i/2 at column block i%2; lane j
-//                       receives 8 consecutive k of column j (four reads = the 32 k of 32x32x64).
+//                       receives 8 consecutive k of column j (four reads = the 32 k a lane holds of a
+//                       16x16x128 operand).
 //
 // MFMA shape.  16-bit inputs use v_mfma_f32_16x16x32, not 32x32x16: with operands held in registers
 // and nothing else running, the matrix pipes of the whole part sustain 1.49 PFLOP/s of 32x32x16 on
 // N(0,1) fp16 data (2.3 PFLOP/s on zeros: the rate depends on the data, i.e. on power), 1.86 PFLOP/s of
 // 16x16x32.  The K loop of this kernel ran at the 32x32x16 figure; on 16x16x32 the GEMM alone is 7-11 %
-// faster.  fp8 inputs use v_mfma_scale_f32_32x32x64_f8f6f4.
+// faster.  fp8 inputs use v_mfma_scale_f32_16x16x128_f8f6f4 for the same reason (3.5 against 4.0 PFLOP/s
+// sustained on N(0,1) e4m3 values; the fp8 GEMM, further from that bound, gained 2 %).
 //
 // Pipeline: LDS holds two stages.  The loads of step kt+1 are issued, woven between the
 // first MFMAs of step kt, into the stage step kt-1 has left.  The step's one barrier
@@ -60,6 +62,9 @@ struct Mfma<fp8e4m3> {
   typedef i32x8 Vec;  // 32 consecutive k of one row / column
   // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled form.
   static TCCL_D f32x16 run(Vec a, Vec b, f32x16 c) { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0); }
+  // 16 x 16 x 128: lane l holds 32 consecutive k (group l / 16) of row / column l % 16 and gets
+  // D[4 * (l / 16) + e][l % 16], e = 0..3.
+  static TCCL_D f32x4 run16(Vec a, Vec b, f32x4 c) { return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0); }
 };
 #endif
 
@@ -360,7 +365,7 @@ struct Gemm256 {
         s.off_b[i] = (uint32_t)(row * g.ldb * kEsz + kc * 16);
       } else if constexpr (kFp8) {
         const int k = 4 * (4 * wave + i) + (lane >> 4);
-        const int c = (lane & 15) ^ (2 * (k & 7));
+        const int c = (lane & 15) ^ (2 * (k & 7)) ^ ((k >> 5) & 1);
         s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
       } else {
         const int k = 2 * (4 * wave + i) + (lane >> 5);
@@ -435,18 +440,19 @@ struct Gemm256 {
         r.b_base0 = (uint32_t)(kAStage256 + (8 * kg + t) * kBPitch + chunk * 16 + (cq & 1) * 8);
       }
     } else {
-      const int half = lane >> 5, l32 = lane & 31, grp = (lane >> 4) & 1;
-      r.a_base = (uint32_t)((wm * 128 + l32) * kARow256);
-      r.a_swz = (uint32_t)((l32 >> 1) & 7);
+      // 16 x 16 x 128 operands: lane l reads row (column) l % 16 of a 16-row block, k group l / 16 (32 k).
+      const int kg = lane >> 4;
+      r.a_base = (uint32_t)((wm * 128 + i16) * kARow256);
+      r.a_swz = (uint32_t)((i16 >> 1) & 7);
       if constexpr (kBKMajor) {
-        r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + l32) * kARow256);  // this lane's row of column block 0
+        r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + i16) * kARow256);  // this lane's row of column block 0
       } else {
-        // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns of k row i/2
-        // (column block i%2) and lane j receives 8 consecutive k of column j.  Four reads
-        // (k + 0, 8, 16, 24) give the 32 consecutive k of v_mfma_f32_32x32x64_f8f6f4.
+        // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns (8 * (i % 2) ..) of k
+        // row i / 2 and lane j receives those 8 k of column j.  Lane group kg covers k rows 32 * kg .. + 31
+        // in four reads (k + 0, 8, 16, 24).
         const int krow = i16 >> 1;
-        const int chunk = (wn * 4 + grp) ^ (2 * krow);
-        r.b_base0 = (uint32_t)(kAStage256 + (32 * half + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
+        const int chunk = (wn * 4) ^ (2 * krow) ^ (kg & 1);
+        r.b_base0 = (uint32_t)(kAStage256 + (32 * kg + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
       }
     }
     return r;
@@ -455,33 +461,35 @@ struct Gemm256 {
   typedef int i32x2 __attribute__((ext_vector_type(2)));
   typedef __attribute__((address_space(3))) i32x2 LdsPair;
 
-  // fp8 operands of k-block kk (64 k): A rows of slab b, B columns of block b.
-  TCCL_D Vec load_a8(const char* stage, const Reader& r, int kk, int b) const {
-    const int half = lane >> 5;
+  // fp8 operands of a K step (128 k, one MFMA deep): the A rows of the 16-row block rb, the B columns of
+  // the 16-column block cb.
+  TCCL_D Vec load_a8(const char* stage, const Reader& r, int rb) const {
+    const int kg = lane >> 4;
     // The two 16-byte chunks of a lane are neighbours under the swizzle (chunk and chunk ^ 1).
     // Both addresses are formed by adding to `stage`: flipping a bit of the pointer itself
     // would hide that it points into LDS, and the load would become a flat load, which
     // waits for every outstanding global load.
-    const uint32_t chunk = ((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz;
-    const char* row = stage + r.a_base + b * 32 * kARow256;
+    const uint32_t chunk = ((uint32_t)(2 * kg)) ^ r.a_swz;
+    const char* row = stage + r.a_base + rb * 16 * kARow256;
     const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
     const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
     typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
     const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(Vec, both);
   }
-  TCCL_D Vec load_b8(const char* stage, const Reader& r, int kk, int b) const {
+  TCCL_D Vec load_b8(const char* stage, const Reader& r, int cb) const {
     if constexpr (kBKMajor) {
-      const int half = lane >> 5;
-      const uint32_t chunk = ((uint32_t)(4 * kk + 2 * half)) ^ r.a_swz;
-      const char* row = stage + r.b_base0 + b * 32 * kARow256;
+      const int kg = lane >> 4;
+      const uint32_t chunk = ((uint32_t)(2 * kg)) ^ r.a_swz;
+      const char* row = stage + r.b_base0 + cb * 16 * kARow256;
       const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
       const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
       typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
       const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(Vec, both);
     }
-    const char* p = stage + (b == 0 ? r.b_base0 : (r.b_base0 ^ 32u)) + 64 * kk * kBPitch;
+    // column block cb: one chunk further on per block (the XOR commutes with the swizzle terms)
+    const char* p = stage + (r.b_base0 ^ (uint32_t)(16 * cb));
     i32x2 q[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) q[t] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsPair*)(p + 8 * t * kBPitch));
@@ -964,43 +972,44 @@ struct Gemm256 {
 
   // fp8 operand registers; they live across K steps.
   struct Frags8 {
-    Vec ring[2], fb[2][2];
+    Vec ring[2], fb[4];
   };
 
-  // One K step of the fp8 path: eight items (k-block kk of 64, A slab bi) of two MFMAs each,
-  // read from `cur` while the next step's operands stream into `nxt` (one pair of loads per
-  // item, items 0..3).  An fp8 operand is 8 registers and an fp8 MFMA lasts twice as long as a
-  // 16-bit one, so the A operand is fetched one item ahead (two register sets); the B
-  // operands of k-block 1 are fetched at item 2.  As in the 16-bit path the step's one barrier
-  // sits inside the step, before item 7: the reads of `cur` are done, the loads into `nxt`
-  // have landed, and item 7 fetches the next step's first operands from `nxt` behind it.
-  // 4096^3 e4m3: 54 us against 62 us with the barrier at the step's end.
+  // One K step of the fp8 path (v_mfma_scale_f32_16x16x128_f8f6f4, 128 k per step): eight items of four
+  // MFMAs, item d = the 16-row block d of the wave tile against its four 16-column blocks, read from
+  // `cur` while the next step's operands stream into `nxt` (one pair of loads per item, items 0..3).
+  // An fp8 operand is 8 registers: the A operand is fetched one item ahead (two register sets), the four
+  // B operands have one set and are reloaded in place during the last item, each as soon as its MFMA is
+  // issued.  As in the 16-bit path the step's one barrier sits inside the step, before item 7: the reads
+  // of `cur` are done, the loads into `nxt` have landed, and item 7 fetches the next step's first
+  // operands from `nxt` behind it.
   TCCL_D void k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                       Frags8& f, PullState& pull, int parity) const {
     pull_issue(pull, pa(), bgw, parity);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int kk = i >> 2, bi = i & 3;
-      const int j = (i + 1) & 7;
-      if (i == 7) {
+    for (int d = 0; d < 8; ++d) {
+      if (d == 7) {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         pull_collect(pull, pa(), bgw, parity);
       }
-      const char* from = i + 1 < 8 ? cur : nxt;
-      f.ring[(i + 1) & 1] = load_a8(from, rd, j >> 2, j & 3);
-      if (i == 2) {
-        f.fb[1][0] = load_b8(cur, rd, 1, 0);
-        f.fb[1][1] = load_b8(cur, rd, 1, 1);
+      const char* from = d + 1 < 8 ? cur : nxt;
+      f.ring[(d + 1) & 1] = load_a8(from, rd, (d + 1) & 7);
+      if (d < 4) issue_piece(nxt, src, kt_load, d);
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) {
+        f32x16& patch = acc[d >> 1][cb >> 1];
+        const int q = 2 * (d & 1) + (cb & 1);
+        f32x4 blk = {patch[4 * q], patch[4 * q + 1], patch[4 * q + 2], patch[4 * q + 3]};
+        blk = Mfma<InT>::run16(f.fb[cb], f.ring[d & 1], blk);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) patch[4 * q + e] = blk[e];
+        if (d == 7) {
+          __builtin_amdgcn_sched_barrier(0);
+          f.fb[cb] = load_b8(nxt, rd, cb);
+        }
       }
-      if (i == 7) {
-        f.fb[0][0] = load_b8(nxt, rd, 0, 0);
-        f.fb[0][1] = load_b8(nxt, rd, 0, 1);
-      }
-      if (i < 4) issue_piece(nxt, src, kt_load, i);
-      acc[bi][0] = Mfma<InT>::run(f.fb[kk][0], f.ring[i & 1], acc[bi][0]);
-      acc[bi][1] = Mfma<InT>::run(f.fb[kk][1], f.ring[i & 1], acc[bi][1]);
       __builtin_amdgcn_sched_barrier(0);
     }
     pull_retire(pull, pa(), bgw, parity);  // the piece this step requested: it arrived before the barrier
@@ -1086,14 +1095,13 @@ struct Gemm256 {
   }
 
   // Where registers 4 * q .. 4 * q + 3 of acc[bi][bj] sit in the 32-row slab bi of the wave tile: row inside
-  // the slab, first of four consecutive columns inside the wave's 64.  fp8 (32 x 32 x 64 MFMA): lane l holds
-  // row l % 32, columns 8 * q + 4 * (l / 32) ..; 16-bit inputs (16 x 16 x 32 MFMA): block q of the patch,
-  // row l % 16 of it, columns 4 * (l / 16) .. .
+  // the slab, first of four consecutive columns inside the wave's 64.  The MFMAs in use (16 x 16 x 32 for
+  // 16-bit inputs, 16 x 16 x 128 for fp8) leave block q of the 32 x 32 patch there: row l % 16 of the block,
+  // columns 4 * (l / 16) .. .
   struct Spot {
     int row, col;
   };
   static TCCL_D Spot acc_spot(int ln, int bj, int q) {
-    if constexpr (kFp8) return Spot{ln & 31, bj * 32 + 8 * q + 4 * (ln >> 5)};
     return Spot{16 * (q >> 1) + (ln & 15), bj * 32 + 16 * (q & 1) + 4 * (ln >> 4)};
   }
 
@@ -1329,9 +1337,9 @@ struct Gemm256 {
     pull_collect(pull, pa(), bgw, 0);  // the counters fetched before this tile (no piece is pending here)
     if constexpr (kFp8) {
       Frags8 f;
-      f.fb[0][0] = load_b8(lds, rd, 0, 0);
-      f.fb[0][1] = load_b8(lds, rd, 0, 1);
-      f.ring[0] = load_a8(lds, rd, 0, 0);
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) f.fb[cb] = load_b8(lds, rd, cb);
+      f.ring[0] = load_a8(lds, rd, 0);
       for (int kt = 0; kt < ksteps; kt += 2) {
         follow_shards(src, kt + 1);
         k_step8(lds, lds1, src, rd, kt + 1, acc, f, pull, 0);
