@@ -538,8 +538,6 @@ struct Gemm256 {
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
     int pend_mask;           // non-zero: a piece was requested and is not yet stored
-    u32x4 seen_pos;          // pull_peek_*(): the lane's LDS state, held for the item between request and use
-    u32x2 seen_pend;
     // The piece itself.  One set of registers: a piece is stored (pull_retire) before the next one is
     // requested, in every path; a second set costs the fused kernels registers they do not have.
     u32x4 piece[1][kPullLoads];
@@ -587,8 +585,6 @@ struct Gemm256 {
     st.probe_val = 0;
 #pragma unroll
     for (int j = 0; j < kPullLoads; ++j) st.piece[0][j] = u32x4{0, 0, 0, 0};
-    st.seen_pos = u32x4{0, 0, 0, 0};
-    st.seen_pend = u32x2{0, 0};
     st.active = pull_offset >= 0 && a->mode != kBgNone && w < kPullWaves;
     st.primed = false;
     st.upr = st.pitch = st.units = 0;
@@ -622,15 +618,6 @@ struct Gemm256 {
   TCCL_D void pull_set_pos(u32x4 pos) const { *(u32x4*)pull_lane() = pos; }
   TCCL_D u32x2 pull_pend() const { return *(const u32x2*)(pull_lane() + 16); }
   TCCL_D void pull_set_pend(u32x2 pend) const { *(u32x2*)(pull_lane() + 16) = pend; }
-  TCCL_D void pull_peek_pend(PullState& st) const {
-    if constexpr (kWithReduce) return;
-    if (st.active) st.seen_pend = pull_pend();
-  }
-  TCCL_D void pull_peek_pos(PullState& st) const {
-    if constexpr (kWithReduce) return;
-    if (st.active) st.seen_pos = pull_pos();
-  }
-
   // (row, col) of this lane's units of piece next_lp, by division: at the start and when a block is finished.
   TCCL_D void pull_locate(PullState& st) const {
     u32x4 pos;
@@ -754,13 +741,12 @@ struct Gemm256 {
   // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.  The
   // piece belongs to the selected block: pull_issue() stores what is pending before it selects
   // another one.
-  template <bool kPeeked = false>
   TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int) const {
     if constexpr (kWithReduce) return false;
     constexpr int slot = 0;
     if (!(st.pend_mask & (1 << slot))) return false;
     const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
-    const u32x2 pend = kPeeked ? st.seen_pend : pull_pend();
+    const u32x2 pend = pull_pend();
 #pragma unroll
     for (int j = 0; j < kPullLoads; ++j)
       if (pend[j] != kNoUnit) st16<kStreaming>(dst, pend[j], st.piece[slot][j]);
@@ -814,7 +800,6 @@ struct Gemm256 {
   // Once per K step: learn about readiness, request the next piece into slot `slot` (its
   // previous piece was stored during the step before).  All control flow here is
   // wavefront-uniform.  Returns whether a piece was requested.
-  template <bool kPeeked = false>
   TCCL_D bool pull_issue(PullState& st, PullPtr a, char* landing, int) const {
     if constexpr (kWithReduce) return false;
     constexpr int slot = 0;
@@ -841,7 +826,7 @@ struct Gemm256 {
     const uint32_t last = first + (uint32_t)(kPieceUnits - 1);
     if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
       const __amdgpu_buffer_rsrc_t src = window(st.src_base);
-      const u32x4 pos = kPeeked ? st.seen_pos : pull_pos();
+      const u32x4 pos = pull_pos();
       u32x2 pend;
       const int ln = lane_now();
 #pragma unroll
@@ -1058,19 +1043,17 @@ struct Gemm256 {
         issue_a(nxt, src, kt_load, d);
         issue_b(nxt, src, kt_load, d);
       }
-      // The pulling lanes' state comes out of LDS an item before it is used: asked for where it is
-      // used, the wait for it would also hold back this wave's MFMAs.
-      if (d == 1) pull_peek_pend(pull);
-      // The piece requested during the step before (it arrived before that step's barrier) is
-      // stored ahead of the next request, so that one set of piece registers serves both.
-      if (d == 2) {
-        pull_retire<true>(pull, pa(), bgw, parity ^ 1);
-        pull_peek_pos(pull);
+      // The background transfer has one place in the step, behind the step's last operand loads (loads
+      // complete in issue order: a request that goes out to the peer's memory ahead of them would hold
+      // all of them back): the piece requested during the step before (it arrived before that step's
+      // barrier) is stored, then the next one is requested into the same registers.  One place, under one
+      // test: every call site splits the step into basic blocks, and where they join the compiler waits
+      // for more than the code needs.  Spread over three items (state read an item ahead of its use) the
+      // same work cost a launch of 4096 x 4096 x 1024 1.3 us more.
+      if (d == 3 && pull.active) {
+        pull_retire(pull, pa(), bgw, parity ^ 1);
+        pull_issue(pull, pa(), bgw, parity);
       }
-      // The next piece is requested behind the step's last operand loads, not ahead of them:
-      // loads complete in issue order, so a request that has to go out to the peer's memory
-      // would hold back every operand load issued after it.
-      if (d == 3) pull_issue<true>(pull, pa(), bgw, parity);
       // acc[rb / 2][cb / 2] holds a 32 x 32 patch as four 16 x 16 blocks: registers 4 * q .. 4 * q + 3 are
       // block q = 2 * (rb % 2) + cb % 2 (acc_spot() is the lane's place in it).
 #pragma unroll
