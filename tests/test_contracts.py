@@ -297,3 +297,13 @@ def test_spill_check_reads_an_assembly_listing():
         "    .vgpr_count:     256",
     ]) + "\n"
     assert list(kernels(asm)) == [(name, 256, 1, 3)]
+
+
+def test_spill_check_tells_reduce_scatter_kernels_apart():
+    """Scratch accesses outside the K loops matter in the reduce-scatter kernels: the check marks them there."""
+    from tileccl_amd.csrc.check_spills import is_reduce
+
+    assert is_reduce("_ZN4tccl15fused256_kernelIDF16_fLb1ELb0ELb0ELb1EEEvNS_12Fused256ArgsE")
+    assert is_reduce("_ZN4tccl15fused256_kernelINS_7fp8e4m3EDF16bLb1ELb0ELb1ELb1EEEvNS_12Fused256ArgsE")
+    assert not is_reduce("_ZN4tccl15fused256_kernelIDF16_DF16_Lb0ELb1ELb0ELb1EEEvNS_12Fused256ArgsE")
+    assert not is_reduce("_ZN4tccl14gemm256_kernelIDF16_fLb1EEEvNS_8GemmArgsENS_5MacroE")

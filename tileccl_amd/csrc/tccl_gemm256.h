@@ -1050,9 +1050,11 @@ struct Gemm256 {
       // test: every call site splits the step into basic blocks, and where they join the compiler waits
       // for more than the code needs.  Spread over three items (state read an item ahead of its use) the
       // same work cost a launch of 4096 x 4096 x 1024 1.3 us more.
-      if (d == 3 && pull.active) {
-        pull_retire(pull, pa(), bgw, parity ^ 1);
-        pull_issue(pull, pa(), bgw, parity);
+      if constexpr (!kWithReduce) {
+        if (d == 3 && pull.active) {
+          pull_retire(pull, pa(), bgw, parity ^ 1);
+          pull_issue(pull, pa(), bgw, parity);
+        }
       }
       // acc[rb / 2][cb / 2] holds a 32 x 32 patch as four 16 x 16 blocks: registers 4 * q .. 4 * q + 3 are
       // block q = 2 * (rb % 2) + cb % 2 (acc_spot() is the lane's place in it).
