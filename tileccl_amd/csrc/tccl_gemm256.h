@@ -16,7 +16,11 @@
 //            lives in slot kc ^ ((r >> 1) & 7).
 //   B stage: natural [k][n]; 16-bit: 512 B per k row, chunk c of row k in slot
 //            c ^ (4 * (k & 3)) ^ (2 * ((k >> 3) & 1)); fp8: 256 B per k row, chunk c of row k in slot
-//            c ^ (2 * (k & 7)) ^ ((k >> 5) & 1).
+//            c ^ (2 * (k & 7)) ^ ((k >> 4) & 1).
+// fp8: the 32 k that lane group kg (lane / 16) holds of a 128-k step are k 16 kg .. 16 kg + 15 and
+// 64 + 16 kg .. 64 + 16 kg + 15, for A and B alike (a sum over k does not care about the order).  A ds_read_b128
+// serves lanes of all four groups in one pass: the groups' chunks kg and kg + 4 fall on different banks,
+// the chunks 2 kg and 2 kg + 1 of 32 consecutive k per group did not (every read took twice as long).
 // A operands are read with ds_read_b128.  B operands are read with the transposing LDS reads
 // of gfx950 (semantics measured on the device, 16 lanes at a time):
 //   ds_read_b64_tr_b16: lane i supplies 4 consecutive n of k row i/4 at column block i%4; lane j
@@ -365,7 +369,7 @@ struct Gemm256 {
         s.off_b[i] = (uint32_t)(row * g.ldb * kEsz + kc * 16);
       } else if constexpr (kFp8) {
         const int k = 4 * (4 * wave + i) + (lane >> 4);
-        const int c = (lane & 15) ^ (2 * (k & 7)) ^ ((k >> 5) & 1);
+        const int c = (lane & 15) ^ (2 * (k & 7)) ^ ((k >> 4) & 1);
         s.off_b[i] = (uint32_t)(k * g.ldb * kEsz + c * 16);
       } else {
         const int k = 2 * (4 * wave + i) + (lane >> 5);
@@ -448,11 +452,11 @@ struct Gemm256 {
         r.b_base0 = (uint32_t)(kAStage256 + (wn * 64 + i16) * kARow256);  // this lane's row of column block 0
       } else {
         // ds_read_b64_tr_b8: within 16 lanes, lane i supplies 8 consecutive columns (8 * (i % 2) ..) of k
-        // row i / 2 and lane j receives those 8 k of column j.  Lane group kg covers k rows 32 * kg .. + 31
-        // in four reads (k + 0, 8, 16, 24).
+        // row i / 2 and lane j receives those 8 k of column j.  Lane group kg covers k rows 16 * kg .. + 15 and
+        // 64 + 16 * kg .. + 15 in four reads (k + 0, 8, 64, 72), the k that load_a8() gives the group.
         const int krow = i16 >> 1;
         const int chunk = (wn * 4) ^ (2 * krow) ^ (kg & 1);
-        r.b_base0 = (uint32_t)(kAStage256 + (32 * kg + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
+        r.b_base0 = (uint32_t)(kAStage256 + (16 * kg + krow) * kBPitch + chunk * 16 + (i16 & 1) * 8);
       }
     }
     return r;
@@ -465,14 +469,14 @@ struct Gemm256 {
   // the 16-column block cb.
   TCCL_D Vec load_a8(const char* stage, const Reader& r, int rb) const {
     const int kg = lane >> 4;
-    // The two 16-byte chunks of a lane are neighbours under the swizzle (chunk and chunk ^ 1).
+    // The two 16-byte chunks of a lane are chunks kg and kg + 4 of the row (chunk and chunk ^ 4 under the swizzle).
     // Both addresses are formed by adding to `stage`: flipping a bit of the pointer itself
     // would hide that it points into LDS, and the load would become a flat load, which
     // waits for every outstanding global load.
-    const uint32_t chunk = ((uint32_t)(2 * kg)) ^ r.a_swz;
+    const uint32_t chunk = ((uint32_t)kg) ^ r.a_swz;
     const char* row = stage + r.a_base + rb * 16 * kARow256;
     const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
-    const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
+    const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 4u) << 4));
     typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
     const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(Vec, both);
@@ -480,10 +484,10 @@ struct Gemm256 {
   TCCL_D Vec load_b8(const char* stage, const Reader& r, int cb) const {
     if constexpr (kBKMajor) {
       const int kg = lane >> 4;
-      const uint32_t chunk = ((uint32_t)(2 * kg)) ^ r.a_swz;
+      const uint32_t chunk = ((uint32_t)kg) ^ r.a_swz;
       const char* row = stage + r.b_base0 + cb * 16 * kARow256;
       const u32x4 lo = *(const u32x4*)(row + (chunk << 4));
-      const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 1u) << 4));
+      const u32x4 hi = *(const u32x4*)(row + ((chunk ^ 4u) << 4));
       typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
       const u32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(Vec, both);
@@ -492,7 +496,7 @@ struct Gemm256 {
     const char* p = stage + (r.b_base0 ^ (uint32_t)(16 * cb));
     i32x2 q[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) q[t] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsPair*)(p + 8 * t * kBPitch));
+    for (int t = 0; t < 4; ++t) q[t] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsPair*)(p + (8 * (t & 1) + 64 * (t >> 1)) * kBPitch));
     i32x8 v;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
