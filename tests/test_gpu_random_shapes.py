@@ -1,6 +1,7 @@
 """Seeded random shapes through the fused all-gather and reduce-scatter against the oracle:
 worlds of 2 to 4 ranks, ragged M / N / K, both GEMM kernels, the three variants, both B layouts,
-several TileGroup sizes.  Moved bytes and two-rank sums are bit-exact; the GEMM and the sums of
+several TileGroup sizes; a second sweep draws larger shapes (K loops of up to 32 steps, several rounds
+of large tiles).  Moved bytes and two-rank sums are bit-exact; the GEMM and the sums of
 three or more ranks (whose fp32 order is pinned elsewhere) are held to the stated tolerances.
 Combinations the library refuses (shards that are not whole tiles, ...) are skipped by their error."""
 
@@ -16,6 +17,19 @@ from tests.gpu_util import bits, into_heap, seeded
 pytestmark = pytest.mark.gpu
 
 CASES_PER_SEED = 120
+
+
+def draw_large(rng):
+    """Shapes with K loops of 2 to 32 steps, several rounds of large tiles and blocks of many pieces."""
+    case = draw(rng)
+    case.update(K=8 * rng.randint(16, 256), N=8 * rng.randint(32, 320))
+    if case["kind"] == "ag":
+        case.update(M=rng.randint(500, 5000))
+    else:
+        shard = rng.choice([512, 768, 1024, 2048]) if rng.random() < 0.8 else rng.randint(300, 1200)
+        case.update(M=shard * case["world"])
+    case["heap"] = 400 << 20
+    return case
 
 
 def draw(rng):
@@ -40,7 +54,7 @@ def run_case(case, seed):
     from tileccl_amd.v2 import FusedGemmAllGather, FusedGemmReduceScatter, SymmetricHeap
 
     world, M, N, K, dtype = case["world"], case["M"], case["N"], case["K"], case["dtype"]
-    heaps = SymmetricHeap.create_all(96 << 20, world)
+    heaps = SymmetricHeap.create_all(case.get("heap", 96 << 20), world)
     try:
         A_cpu, B_cpu = seeded((M, K), seed, dtype), seeded((K, N), seed + 1, dtype, scale=K**-0.5)
         common = dict(macro_tile=case["macro"], tau_min_bytes=case["tau"], group_m=case["group_m"], block_m=case["block_m"])
@@ -126,3 +140,17 @@ def test_random_shapes(lib, seed):
         except AssertionError as e:
             raise AssertionError(f"case {i} of seed {seed}: {case}: {e}") from e
     assert checked >= CASES_PER_SEED // 2  # most draws are supported combinations
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_large_shapes(lib, seed):
+    rng = random.Random(seed)
+    checked = 0
+    for i in range(40):
+        case = draw_large(rng)
+        try:
+            checked += 1 if run_case(case, 1000 * seed + i) else 0
+        except AssertionError as e:
+            raise AssertionError(f"case {i} of seed {seed}: {case}: {e}") from e
+    assert checked >= 20
+
