@@ -974,7 +974,6 @@ struct Gemm256 {
   // operands from `nxt` behind it.
   TCCL_D void k_step8(const char* cur, char* nxt, const Source& src, const Reader& rd, int kt_load, f32x16 (&acc)[4][2],
                       Frags8& f, PullState& pull, int parity) const {
-    pull_issue(pull, pa(), bgw, parity);
 #pragma unroll
     for (int d = 0; d < 8; ++d) {
       if (d == 7) {
@@ -986,6 +985,14 @@ struct Gemm256 {
       const char* from = d + 1 < 8 ? cur : nxt;
       f.ring[(d + 1) & 1] = load_a8(from, rd, (d + 1) & 7);
       if (d < 4) issue_piece(nxt, src, kt_load, d);
+      // The background transfer's one place in the step, as in the 16-bit path: behind the step's last
+      // operand loads, the piece of the step before stored first, the next one requested into its registers.
+      if constexpr (!kWithReduce) {
+        if (d == 3 && pull.active) {
+          pull_retire(pull, pa(), bgw, parity ^ 1);
+          pull_issue(pull, pa(), bgw, parity);
+        }
+      }
 #pragma unroll
       for (int cb = 0; cb < 4; ++cb) {
         f32x16& patch = acc[d >> 1][cb >> 1];
@@ -1001,7 +1008,6 @@ struct Gemm256 {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    pull_retire(pull, pa(), bgw, parity);  // the piece this step requested: it arrived before the barrier
   }
 
   // One K step of the 16-bit path (v_mfma_f32_16x16x32): eight items of eight MFMAs each, read from `cur`
