@@ -373,6 +373,24 @@ int launch_fused256(int in_dtype, int out_dtype, const Fused256Args& f, int wgs,
   return launch_status(rc, in_dtype, out_dtype);
 }
 
+// How the background transfer addresses the 16-byte units of a block (PullArgs::row_units and what follows):
+// rows of `upr` units, `pitch` bytes apart on the destination side and `src_pitch` on the source side.  Rows that
+// follow each other without gaps on both sides are one long row.  The kernel divides by multiplying:
+// u / d = mulhi(u, magic) >> shift with shift = floor(log2 d), magic = ceil(2^(32 + shift) / d), which fits 32
+// bits for every d that is not a power of two and is exact for u < 2^31 (the error term u * (magic * d -
+// 2^(32 + shift)) stays below 2^(32 + shift)); a power of two is magic = 0 and a plain shift.
+void set_row_divider(tccl::PullArgs* p, uint32_t upr, uint32_t pitch, uint32_t src_pitch) {
+  const bool flat = pitch == upr * 16u && src_pitch == upr * 16u;
+  const uint32_t d = flat ? (p->units > 0 ? p->units : 1u) : upr;
+  p->row_units = d;
+  p->row_pitch = pitch;
+  p->src_row_pitch = src_pitch;
+  uint32_t shift = 0;
+  while ((2ull << shift) <= d) ++shift;  // floor(log2 d)
+  p->row_shift = shift;
+  p->row_magic = (d & (d - 1)) == 0 ? 0u : (uint32_t)((((uint64_t)1 << (32 + shift)) + d - 1) / d);
+}
+
 // The pull half of a TileGroup all-gather, as the large-tile K loop performs it in the
 // background.  Returns false when there is nothing of the kind to do (the communication role
 // after the last tile then does it).
@@ -404,6 +422,7 @@ bool build_background(const tccl::CommArgs& c, tccl::PullArgs* p) {
   p->upr = (uint32_t)(row_bytes / 16);
   p->units = (uint32_t)p->block_rows * p->upr;
   p->pieces = (int)((p->units + tccl::kPieceUnits - 1) / tccl::kPieceUnits);
+  set_row_divider(p, p->upr, p->pitch, p->pitch);
   p->counter = by_tile ? c.locks : c.counter;
   p->row_ends = c.row_ends;
   p->tile_counts = c.tile_counts;
@@ -547,6 +566,7 @@ void build_gather_background(const tccl_gemm_desc* d, const GatherSpec& gs, cons
   p->upr = (uint32_t)((int64_t)gs.k_shard * esz / 16);
   p->units = (uint32_t)d->M * p->upr;
   p->pieces = (int)((p->units + tccl::kPieceUnits - 1) / tccl::kPieceUnits);
+  set_row_divider(p, p->upr, p->pitch, p->src_pitch);
   p->epoch = 1;
   p->fault = c.fault;
   p->spin_ticks = c.spin_ticks;

@@ -71,11 +71,17 @@ struct OperandOrigin {
 TCCL_HD OperandOrigin operand_origin(const GemmArgs& g, int row0, int col0) {
   OperandOrigin o;
   if (g.wrap_rows > 0) {
-    const int q = row0 / g.wrap_rows;
-    o.a_row = row0 - q * g.wrap_rows;
-    o.a_rows = g.wrap_rows;
+    int wrap_rows = g.wrap_rows;
+#if defined(__HIP_DEVICE_COMPILE__)
+    // Hidden from the optimiser: it would otherwise prepare this division (a reciprocal and its
+    // corrections) at the kernel's start for every launch, column shards or not.
+    asm volatile("" : "+s"(wrap_rows));
+#endif
+    const int q = row0 / wrap_rows;
+    o.a_row = row0 - q * wrap_rows;
+    o.a_rows = wrap_rows;
     o.b_col = col0 + q * g.N;
-    o.b_cols = (g.M / g.wrap_rows) * g.N;
+    o.b_cols = (g.M / wrap_rows) * g.N;
   } else {
     o.a_row = row0;
     o.a_rows = g.M;

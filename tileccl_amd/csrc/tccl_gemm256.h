@@ -167,6 +167,11 @@ struct PullArgs {
   int64_t spin_ticks;
   int64_t word_stride;         // as in CommArgs: 0 = a peer's counters sit in its heap slice
   uint32_t src_pitch;          // kBgGatherCols: bytes per row of a shard (`pitch` is the workspace's)
+  // Addressing of a unit u of a block: row = u / row_units, byte offset = row * row_pitch + (u - row * row_units) * 16
+  // (source: src_row_pitch).  The division is a multiplication: row = row_magic ? mulhi(u, row_magic) >> row_shift
+  // : u >> row_shift (set_row_divider() in tccl_api.hip; exact for u < 2^31).  A block whose rows follow each
+  // other without gaps is described as one row of `units` units.
+  uint32_t row_units, row_magic, row_shift, row_pitch, src_row_pitch;
   // Tile-by-tile readiness (S1): `counter` points at the locks, a "group" is a pair of plan-tile
   // rows, complete once every lock of both rows has reached `epoch`; n_groups = ceil(tile_rows / 2).
   int tile_mode;
@@ -195,8 +200,6 @@ constexpr int kBgWordBytes = 8 * 256;                   // a fetched counter wor
 // alone, two 16-byte units per lane and step, so that its bookkeeping runs once per 2 KiB and
 // only where it is covered.
 constexpr int kPullWaves = 4;                           // wavefronts of a workgroup that pull
-constexpr int kPullLaneBytes = 32;                      // per-lane pull state kept in LDS (see PullLane)
-constexpr int kPullStateBytes = kPullWaves * 64 * kPullLaneBytes;
 constexpr int kPullLoads = 2;                           // 16-byte units per lane and piece
 constexpr int kPieceUnits = 64 * kPullLoads;            // units per piece
 
@@ -274,7 +277,6 @@ struct Gemm256 {
   char* lds;   // stage 0 (also the epilogue's staging area)
   char* lds1;  // stage 1
   char* bgw;   // landing words of the background transfer's counter fetches
-  char* pls;   // per-lane state of the pulling wavefronts (kPullStateBytes of LDS; nullptr: nothing pulls)
   const int tid, lane, wave, wm, wn;
   // A per-lane value the optimiser must treat as new at this point (blocks hoisting of what is derived from it).
   static TCCL_D int fresh(int v) {
@@ -294,8 +296,8 @@ struct Gemm256 {
 
 
   TCCL_D Gemm256(const GemmArgs& args, int pull_args_offset, int push_args_offset, int reduce_args_offset, char* stage0,
-                 char* stage1, char* landing_words, int gather_args_offset = -1, char* pull_lane_state = nullptr)
-      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), gather_offset(gather_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), pls(pull_lane_state), tid(threadIdx.x), lane(threadIdx.x & 63),
+                 char* stage1, char* landing_words, int gather_args_offset = -1)
+      : g(args), pull_offset(pull_args_offset), push_offset(push_args_offset), reduce_offset(reduce_args_offset), gather_offset(gather_args_offset), lds(stage0), lds1(stage1), bgw(landing_words), tid(threadIdx.x), lane(threadIdx.x & 63),
         // the wavefront's number is the same in all its lanes: held in a scalar register, and with it the LDS
         // addresses its loads land at (kept per lane they cost eight registers and a readfirstlane per load)
         wave(__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)), wm(__builtin_amdgcn_readfirstlane(threadIdx.x >> 8)),
@@ -350,6 +352,11 @@ struct Gemm256 {
   TCCL_D Source make_source(int row0, int col0) const {
     constexpr int kEsz = sizeof(InT);
     Source s;
+    // The lane's number is taken afresh: derived from the member, the offsets below are the same for every
+    // tile, get computed once at the kernel's start and, in the kernels that sit at the register limit, are
+    // parked in scratch memory through the K loops; reloading them between a tile's first operand requests
+    // made each reload wait for the requests ahead of it (three trips to memory in a row, 2 us per tile).
+    const int lane = lane_now();
     const OperandOrigin o = operand_origin(g, row0, col0);
     const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
     const InT* B = (const InT*)g.B + (kBKMajor ? (int64_t)o.b_col * g.ldb : (int64_t)o.b_col);
@@ -541,7 +548,7 @@ struct Gemm256 {
     int32_t need;            // epoch * tile_counts[gidx]: what the counters of group gidx must reach
     uint32_t group_units;    // ready_units once group gidx is complete
     int backoff;             // K steps to let pass before the counters are fetched again
-    int pend_mask;           // non-zero: a piece was requested and is not yet stored
+    int pend_lp;             // piece of the selected block that was requested and is not yet stored (-1: none)
     // The piece itself.  One set of registers: a piece is stored (pull_retire) before the next one is
     // requested, in every path; a second set costs the fused kernels registers they do not have.
     u32x4 piece[1][kPullLoads];
@@ -550,13 +557,11 @@ struct Gemm256 {
     // there, it is older than every operand fetch that follows, so using it never waits for those.
     int32_t probe_val;
     // What the per-step code needs from PullArgs, kept in registers (reading a field through
-    // the argument block is a scalar load plus a wait that also drains the operand fetches),
-    // and piece positions that advance without divisions.
+    // the argument block is a scalar load plus a wait that also drains the operand fetches).
     bool active;
-    bool primed;             // the first counters have been requested (pull_prime)
-    uint32_t upr, pitch, units;
+    uint32_t units;
     int pieces, slots, n_groups;
-    uint32_t adv_row, adv_col;   // what `stride` pieces add to (row, col)
+    uint32_t row_units, row_magic, row_shift, row_pitch;
   };
 
   // Values that are the same in every lane but that the compiler cannot prove so (loaded
@@ -585,66 +590,46 @@ struct Gemm256 {
     st.need = 0;
     st.group_units = 0;
     st.backoff = 0;
-    st.pend_mask = 0;
+    st.pend_lp = -1;
     st.probe_val = 0;
 #pragma unroll
     for (int j = 0; j < kPullLoads; ++j) st.piece[0][j] = u32x4{0, 0, 0, 0};
     st.active = pull_offset >= 0 && a->mode != kBgNone && w < kPullWaves;
-    st.primed = false;
-    st.upr = st.pitch = st.units = 0;
+    st.units = 0;
     st.pieces = st.slots = st.n_groups = 0;
-    st.adv_row = st.adv_col = 0;
+    st.row_units = 1;
+    st.row_magic = st.row_shift = st.row_pitch = 0;
     if (st.active) {
-      st.upr = a->upr;
-      st.pitch = a->pitch;
       st.units = a->units;
       st.pieces = a->pieces;
       st.slots = a->slots;
       st.n_groups = a->n_groups;
-      const uint32_t adv = (uint32_t)st.stride * (uint32_t)kPieceUnits;
-      st.adv_row = adv / st.upr;
-      st.adv_col = adv - st.adv_row * st.upr;
+      st.row_units = a->row_units;
+      st.row_magic = a->row_magic;
+      st.row_shift = a->row_shift;
+      st.row_pitch = a->row_pitch;
       pull_normalise(st, a);
-      pull_locate(st);
     }
     return st;
   }
 
-  // What a pulling lane carries from K step to K step besides the piece itself lives in LDS, not in
-  // registers (the fused kernels have none to spare, and a register spilled to scratch memory comes back
-  // through the same queue as the operand loads: a reload inside the K loop waits for all of them).
-  //   pos  = { row[0], row[1], col[0], col[1] }: row / unit-in-row of this lane's units of piece next_lp
-  //   pend = { off[0], off[1] }: byte offsets of the pending piece's units inside the block; kNoUnit: the
-  //          unit does not exist (a block's last piece may be short)
-  static_assert(kPullLoads == 2, "PullLane holds two units per lane");
-  TCCL_D char* pull_lane() const { return pls + (wave * 64 + lane_now()) * kPullLaneBytes; }  // wave < kPullWaves
-  TCCL_D u32x4 pull_pos() const { return *(const u32x4*)pull_lane(); }
-  TCCL_D void pull_set_pos(u32x4 pos) const { *(u32x4*)pull_lane() = pos; }
-  TCCL_D u32x2 pull_pend() const { return *(const u32x2*)(pull_lane() + 16); }
-  TCCL_D void pull_set_pend(u32x2 pend) const { *(u32x2*)(pull_lane() + 16) = pend; }
-  // (row, col) of this lane's units of piece next_lp, by division: at the start and when a block is finished.
-  TCCL_D void pull_locate(PullState& st) const {
-    u32x4 pos;
-#pragma unroll
-    for (int j = 0; j < kPullLoads; ++j) {
-      const uint32_t u = (uint32_t)st.next_lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane_now());
-      pos[j] = u / st.upr;
-      pos[2 + j] = u - pos[j] * st.upr;
-    }
-    pull_set_pos(pos);
-  }
-  // The same after next_lp += stride.
-  TCCL_D void pull_advance(PullState& st, u32x4 pos) const {
-#pragma unroll
-    for (int j = 0; j < kPullLoads; ++j) {
-      pos[j] += st.adv_row;
-      pos[2 + j] += st.adv_col;
-      if (pos[2 + j] >= st.upr) {
-        pos[2 + j] -= st.upr;
-        ++pos[j];
-      }
-    }
-    pull_set_pos(pos);
+  // Where this lane's unit j of piece lp lies inside a block: byte offsets on the destination and the source
+  // side (kNoUnit / the block's first unit for lanes beyond the block's end: their stores fall outside the
+  // buffer window and are dropped, their loads touch a unit that exists).  A handful of vector instructions
+  // from three scalars, formed where a piece is requested and again where it is stored: whatever a pulling
+  // lane carries from K step to K step besides the piece itself costs registers that the fused kernels do
+  // not have (kept in LDS instead, its reads and their waits made the per-step code several times as long).
+  static constexpr uint32_t kNoUnit = 0xffffffffu;
+  TCCL_D void pull_where(const PullState& st, PullPtr a, int lp, int j, int ln, uint32_t& to, uint32_t& from) const {
+    const uint32_t u = (uint32_t)lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + ln);
+    const bool valid = u < st.units;
+    const uint32_t uu = valid ? u : 0u;
+    const uint32_t row = st.row_magic ? (__umulhi(uu, st.row_magic) >> st.row_shift) : (uu >> st.row_shift);
+    const uint32_t col = uu - row * st.row_units;
+    const uint32_t off = row * st.row_pitch + col * 16u;
+    to = valid ? off : kNoUnit;
+    from = off;
+    if constexpr (kGatherA) from = row * a->src_row_pitch + col * 16u;
   }
 
   // Fetch the first counters in the first tile's prologue, so that the first K step can
@@ -673,15 +658,6 @@ struct Gemm256 {
       st.next_lp -= a->pieces;
       ++st.next_slot;
     }
-  }
-
-  // Row and 16-byte unit inside the row of this lane's unit j of piece lp (row 0, unit 0 for idle lanes).
-  TCCL_D void pull_unit(PullPtr a, int lp, int j, bool& valid, uint32_t& row, uint32_t& col) const {
-    const uint32_t u = (uint32_t)lp * (uint32_t)kPieceUnits + (uint32_t)(64 * j + lane);
-    valid = u < a->units;
-    const uint32_t uu = valid ? u : 0u;  // idle lanes touch the block's first unit and store nothing
-    row = uu / a->upr;
-    col = uu - row * a->upr;
   }
 
   TCCL_D uint32_t pull_last_unit(PullPtr a, int lp) const {
@@ -740,21 +716,20 @@ struct Gemm256 {
     }
   }
 
-  static constexpr uint32_t kNoUnit = 0xffffffffu;
-
-  // Store the piece held in slot `slot`, if any.  Returns whether a store was issued.  The
-  // piece belongs to the selected block: pull_issue() stores what is pending before it selects
-  // another one.
+  // Store the piece that is pending, if any.  Returns whether a store was issued.  The piece belongs
+  // to the selected block: pull_issue() stores what is pending before it selects another one.
   TCCL_D bool pull_retire(PullState& st, PullPtr a, const char* landing, int) const {
     if constexpr (kWithReduce) return false;
-    constexpr int slot = 0;
-    if (!(st.pend_mask & (1 << slot))) return false;
+    if (st.pend_lp < 0) return false;
     const __amdgpu_buffer_rsrc_t dst = window(st.dst_base);
-    const u32x2 pend = pull_pend();
+    const int ln = lane_now();
 #pragma unroll
-    for (int j = 0; j < kPullLoads; ++j)
-      if (pend[j] != kNoUnit) st16<kStreaming>(dst, pend[j], st.piece[slot][j]);
-    st.pend_mask &= ~(1 << slot);
+    for (int j = 0; j < kPullLoads; ++j) {
+      uint32_t to, from;
+      pull_where(st, a, st.pend_lp, j, ln, to, from);
+      st16<kStreaming>(dst, to, st.piece[0][j]);
+    }
+    st.pend_lp = -1;
     return true;
   }
 
@@ -806,7 +781,6 @@ struct Gemm256 {
   // wavefront-uniform.  Returns whether a piece was requested.
   TCCL_D bool pull_issue(PullState& st, PullPtr a, char* landing, int) const {
     if constexpr (kWithReduce) return false;
-    constexpr int slot = 0;
     if (!st.active) return false;
     if (st.probe_group >= 0) {
       const int g = st.probe_group;
@@ -820,7 +794,7 @@ struct Gemm256 {
     }
     if (st.next_slot >= st.slots) return false;
     if (st.next_slot != st.slot) {
-      pull_retire(st, a, landing, slot);  // a piece still pending belongs to the block being left
+      pull_retire(st, a, landing, 0);  // a piece still pending belongs to the block being left
       pull_select(st, a, st.next_slot);
       pull_probe(st, a, landing);
       return false;
@@ -830,27 +804,16 @@ struct Gemm256 {
     const uint32_t last = first + (uint32_t)(kPieceUnits - 1);
     if ((last < st.units ? last : st.units - 1u) < st.ready_units) {
       const __amdgpu_buffer_rsrc_t src = window(st.src_base);
-      const u32x4 pos = pull_pos();
-      u32x2 pend;
       const int ln = lane_now();
 #pragma unroll
       for (int j = 0; j < kPullLoads; ++j) {
-        const bool valid = first + (uint32_t)(64 * j + ln) < st.units;
-        const uint32_t off = valid ? pos[j] * st.pitch + pos[2 + j] * 16u : 0u;  // idle lanes touch the block's first unit
-        uint32_t from = off;
-        if constexpr (kGatherA) from = valid ? pos[j] * a->src_pitch + pos[2 + j] * 16u : 0u;
-        st.piece[slot][j] = ld16<kCoherent>(src, from);
-        pend[j] = valid ? off : kNoUnit;
+        uint32_t to, from;
+        pull_where(st, a, st.next_lp, j, ln, to, from);
+        st.piece[0][j] = ld16<kCoherent>(src, from);
       }
-      pull_set_pend(pend);
-      st.pend_mask |= 1 << slot;
+      st.pend_lp = st.next_lp;
       st.next_lp += st.stride;
-      if (st.next_lp >= st.pieces) {  // block finished: rare, may divide
-        pull_normalise(st, a);
-        pull_locate(st);
-      } else {
-        pull_advance(st, pos);
-      }
+      if (st.next_lp >= st.pieces) pull_normalise(st, a);  // block finished: rare
       return true;
     }
     return false;
@@ -923,12 +886,9 @@ struct Gemm256 {
           if (ok) {
 #pragma unroll
             for (int j = 0; j < kPullLoads; ++j) {
-              bool valid;
-              uint32_t row, col;
-              pull_unit(a, lp, j, valid, row, col);
-              const uint32_t o = row * a->pitch + col * 16u;
-              v[k][j] = ld16<kCoherent>(src, kGatherA ? row * a->src_pitch + col * 16u : o);
-              off[k][j] = valid ? o : kNoUnit;
+              uint32_t from;
+              pull_where(st, a, lp, j, lane, off[k][j], from);
+              v[k][j] = ld16<kCoherent>(src, from);
             }
             loaded[k] = true;
             n = k + 1;
@@ -1089,6 +1049,23 @@ struct Gemm256 {
     }
   }
 
+  // A finished macro tile whose signal is still owed.  What the signal needs from memory (the TileGroup of
+  // each plan tile under the macro tile) is fetched when the tile is finished, through the scalar path and
+  // ahead of the wait for the tile's stores: looked up behind that wait, by the publishing lane and one plan
+  // tile after the other, the table reads were a chain of trips to memory (1.7 us at 4096 x 4096 x 1024)
+  // between the moment the last store had landed and the moment the signal went out.
+  struct Owed {
+    int where;        // (macro row << 16) | macro column; < 0: nothing owed
+    int32_t tile[4];  // plan tile ids under the macro tile (-1: outside the grid)
+    int32_t gid[4];   // their TileGroups (group mode)
+  };
+  static TCCL_D Owed nothing_owed() {
+    Owed o;
+    o.where = -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o.tile[i] = o.gid[i] = -1;
+    return o;
+  }
   // Where registers 4 * q .. 4 * q + 3 of acc[bi][bj] sit in the 32-row slab bi of the wave tile: row inside
   // the slab, first of four consecutive columns inside the wave's 64.  The MFMAs in use (16 x 16 x 32 for
   // 16-bit inputs, 16 x 16 x 128 for fp8) leave block q of the 32 x 32 patch there: row l % 16 of the block,
@@ -1301,8 +1278,19 @@ struct Gemm256 {
   // `unpublished` carries a finished tile whose signal is still owed (-1: none): instead of
   // waiting for its stores to land right after its epilogue, the next tile's prologue, which
   // has to wait for its first operands anyway, publishes it.
-  TCCL_D void macro_tile(const SignalArgs& s, int mm, int mn, PullState& pull, int& unpublished) const {
+  // `ahead`: `src` describes this tile and its first operands are already requested (a workgroup's first tile: run()).
+  TCCL_D void macro_tile(const SignalArgs& s, int mm, int mn, PullState& pull, Owed& unpublished, Source& src, bool ahead) const {
     const int row0 = mm * kMacro, col0 = mn * kMacro;
+    if (!ahead) {
+      src = make_source(row0, col0);
+      __syncthreads();  // the previous tile's epilogue has left LDS
+#pragma unroll
+      for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
+    }
+    // K steps are taken in pairs so that each call names its two stages statically and the
+    // accumulators flow through one straight loop body.  An odd step count is rounded up: the
+    // extra step (like the final look-ahead load) lies wholly past K and reads zeros.
+    const int ksteps = ((g.K + kStepK - 1) / kStepK + 1) & ~1;
     f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -1310,22 +1298,7 @@ struct Gemm256 {
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    Source src = make_source(row0, col0);
     const Reader rd = make_reader();
-    // K steps are taken in pairs so that each call names its two stages statically and the
-    // accumulators flow through one straight loop body.  An odd step count is rounded up: the
-    // extra step (like the final look-ahead load) lies wholly past K and reads zeros.
-    const int ksteps = ((g.K + kStepK - 1) / kStepK + 1) & ~1;
-    __syncthreads();  // the previous tile's epilogue has left LDS
-#pragma unroll
-    for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
-    // The first counters are requested behind the first operands: the chain of dependent
-    // scalar loads that leads to them (slice bases, tile counts) then runs while those are in flight.
-    if (!pull.primed) {
-      pull_prime(pull, pa(), bgw);
-      pull.primed = true;
-    }
     wait_vmem();  // the first operands are there, and so is everything the previous tile stored
     __syncthreads();
     publish_owed(s, unpublished);
@@ -1369,20 +1342,18 @@ struct Gemm256 {
         const bool for_peer = !kFp8 && owner != ra->rank && ra->emulate_peer && ra->world == 2;
         if ((owner == ra->rank || for_peer) && reduce_wait(ra, s, mm, mn)) {
           epilogue_reduce(ra, row0, col0, acc, owner, for_peer);
-          unpublished = (mm << 16) | mn;
+          unpublished = publish_lookup(s, mm, mn);
           return;
         }
       }
     }
     epilogue<kPolicy>(row0, col0, acc);
     if constexpr (kPolicy != 0) {
-      if constexpr (!kWithReduce) {
-        unpublished = (mm << 16) | mn;
-        return;
-      }
+      unpublished = publish_lookup(s, mm, mn);
+      if constexpr (!kWithReduce) return;
       wait_vmem();  // the tile's write-through stores have landed
       __syncthreads();
-      if (tid == 0 && s.mode != kSignalNone) publish(s, mm, mn);
+      publish_owed(s, unpublished);
       if constexpr (kWithReduce) {
         const ReducePtr ra = late_kernarg_ptr<ReduceArgs>(reduce_offset);
         if (ra->active) {
@@ -1393,11 +1364,52 @@ struct Gemm256 {
     }
   }
 
+  TCCL_D Owed publish_lookup(const SignalArgs& s, int mm, int mn) const {
+    Owed o = nothing_owed();
+    o.where = (mm << 16) | mn;
+    if (s.mode == kSignalNone) return o;
+    const int per_m = kMacro / g.block_m, per_n = kMacro / g.block_n;  // 1 or 2 each
+    const int tm0 = mm * per_m, tn0 = mn * per_n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int dm = i >> 1, dn = i & 1;
+      const int tm = tm0 + dm, tn = tn0 + dn;
+      if (dm < per_m && dn < per_n && tm < g.tile_rows && tn < g.tile_cols) o.tile[i] = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
+    }
+    if (s.mode != kSignalTile) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (o.tile[i] >= 0) o.gid[i] = table(s.group_table, o.tile[i]);
+    }
+    return o;
+  }
+
   // Call behind a wait for this wavefront's stores and a barrier: every store of the owed tile has landed.
-  TCCL_D void publish_owed(const SignalArgs& s, int& unpublished) const {
-    if (unpublished < 0) return;
-    if (tid == 0 && s.mode != kSignalNone) publish(s, unpublished >> 16, unpublished & 0xffff);
-    unpublished = -1;
+  // Plan tiles of one TileGroup are summed up and the group gets one add (concurrent adds to one word serialise).
+  TCCL_D void publish_owed(const SignalArgs& s, Owed& o) const {
+    if (o.where < 0) return;
+    if (tid == 0 && s.mode != kSignalNone) {
+      if (s.mode == kSignalTile) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (o.tile[i] >= 0) tile_publish(s.locks, o.tile[i], s.epoch);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (o.tile[i] < 0) continue;
+          bool counted = false;  // an earlier plan tile of the same group has taken this one along
+          int count = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (o.tile[j] < 0 || o.gid[j] != o.gid[i]) continue;
+            if (j < i) counted = true;
+            ++count;
+          }
+          if (!counted) add_to_group(s, o.gid[i], count);
+        }
+      }
+    }
+    o.where = -1;
   }
 
   // Are the peers' partials of the plan tiles under macro tile (mm, mn) published?  One lane
@@ -1513,31 +1525,6 @@ struct Gemm256 {
     }
   }
 
-  // Plan tiles of one row share a TileGroup, so the group counts are summed up here and
-  // each group gets one add (concurrent adds to one word serialise).
-  TCCL_D void publish(const SignalArgs& s, int mm, int mn) const {
-    const int tm0 = mm * (kMacro / g.block_m), tn0 = mn * (kMacro / g.block_n);
-    int group = -1, count = 0;
-    for (int dm = 0; dm < kMacro / g.block_m; ++dm)
-      for (int dn = 0; dn < kMacro / g.block_n; ++dn) {
-        const int tm = tm0 + dm, tn = tn0 + dn;
-        if (tm >= g.tile_rows || tn >= g.tile_cols) continue;
-        const int tile_id = tile_id_of(tm, tn, g.tile_rows, g.tile_cols, g.group_m);
-        if (s.mode == kSignalTile) {
-          tile_publish(s.locks, tile_id, s.epoch);
-          continue;
-        }
-        const int gi = s.group_table[tile_id];
-        if (gi != group && count > 0) {
-          add_to_group(s, group, count);
-          count = 0;
-        }
-        group = gi;
-        ++count;
-      }
-    if (count > 0) add_to_group(s, group, count);
-  }
-
   TCCL_D void add_to_group(const SignalArgs& s, int group, int count) const {
     // The previous value is only needed for the trace stamp.  Without it the add is issued and
     // forgotten: waiting for the old value costs a round trip that grows with the number of
@@ -1550,26 +1537,65 @@ struct Gemm256 {
     }
   }
 
+  // n / d for n >= 0, d > 0.  The divisors of the slot -> tile map are powers of two for most shapes (a
+  // shift), and an unsigned division is half the instructions of a signed one: the map runs at the very
+  // start of a kernel, where one wavefront per SIMD executes a few hundred scalar instructions with
+  // nothing to overlap them, ahead of the first operand request.
+  static TCCL_D uint32_t quotient(uint32_t n, uint32_t d) {
+    if ((d & (d - 1)) == 0) return n >> (31 - __builtin_clz(d));
+    // The divisor is hidden from the optimiser here: it would otherwise form the reciprocals of every
+    // divisor once, ahead of the tile loop (i.e. at the kernel's start), whether this path is taken or not.
+    asm volatile("" : "+s"(d));
+    return n / d;
+  }
+  // tile_for_slot() followed by macro_coords() and the row shift, in that arithmetic.
   static TCCL_D TileCoord tile_of_slot(int slot, int total, const Macro& m) {
-    const int id = tile_for_slot(slot, total, m.xcds, m.span);
-    TileCoord c = macro_coords(id, m);
-    c.m += m.row_shift;
+    const uint32_t block = (uint32_t)(m.xcds * m.span);
+    uint32_t id = (uint32_t)slot;
+    const uint32_t base = quotient(id, block) * block;
+    if (m.xcds > 1 && base + block <= (uint32_t)total) {
+      const uint32_t r = id - base, q = quotient(r, (uint32_t)m.xcds);
+      id = base + (r - q * (uint32_t)m.xcds) * (uint32_t)m.span + q;
+    }
+    const uint32_t per_band = (uint32_t)(m.rows_per_band * m.cols);
+    const uint32_t band = quotient(id, per_band);
+    const uint32_t first = band * (uint32_t)m.rows_per_band;
+    const uint32_t left = (uint32_t)m.rows - first;
+    const uint32_t height = left < (uint32_t)m.rows_per_band ? left : (uint32_t)m.rows_per_band;
+    const uint32_t within = id - band * per_band;
+    const uint32_t col = quotient(within, height);
+    TileCoord c;
+    c.m = (int)(first + (within - col * height)) + m.row_shift;
+    c.n = (int)col;
     if (c.m >= m.rows) c.m -= m.rows;
     return c;
   }
 
   TCCL_D void run(const SignalArgs& s, const Macro& m, int wg, int num_wgs) const {
     const int total = m.rows * m.cols;
+    // A workgroup's first operand requests go out before anything else it sets up: a kernel's start is
+    // a few hundred scalar and address instructions of one wavefront per SIMD with nothing to overlap
+    // them, followed by a trip to memory, and only what those requests themselves need should come
+    // ahead of that trip.  The rest (the background transfer's state and its first counter fetch, which
+    // is a chain of dependent scalar loads; whatever the optimiser computes once for all tiles) runs
+    // while the operands are in flight.  LDS is free at this point: no barrier.
+    // (A workgroup beyond the last tile requests some tile's operands and never uses them.)
+    const TileCoord c0 = tile_of_slot(wg < total ? wg : total - 1, total, m);
+    Source src = make_source(c0.m * kMacro, c0.n * kMacro);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_piece(lds, src, 0, i);
+    __builtin_amdgcn_sched_barrier(0);
     PullState pull = pull_begin(pa(), wg, num_wgs);
-    int unpublished = -1;
+    pull_prime(pull, pa(), bgw);
+    Owed unpublished = nothing_owed();
     for (int slot = wg; slot < total; slot += num_wgs) {
       const TileCoord c = tile_of_slot(slot, total, m);
       if (s.mode == kSignalNone && push_offset < 0)
-        macro_tile<0>(s, c.m, c.n, pull, unpublished);
+        macro_tile<0>(s, c.m, c.n, pull, unpublished, src, slot == wg);
       else
-        macro_tile<kCoherent>(s, c.m, c.n, pull, unpublished);
+        macro_tile<kCoherent>(s, c.m, c.n, pull, unpublished, src, slot == wg);
     }
-    if (unpublished >= 0) {  // the last tile: nothing follows that would wait for its stores
+    if (unpublished.where >= 0) {  // the last tile: nothing follows that would wait for its stores
       wait_vmem();
       __syncthreads();
       publish_owed(s, unpublished);

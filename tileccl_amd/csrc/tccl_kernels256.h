@@ -55,12 +55,11 @@ __global__ __launch_bounds__(512, 2) void fused256_kernel(Fused256Args f) {
   __shared__ __attribute__((aligned(16))) char stage0[kStage256];
   __shared__ __attribute__((aligned(16))) char stage1[kStage256];
   __shared__ __attribute__((aligned(16))) char landing_words[kBgWordBytes];
-  __shared__ __attribute__((aligned(16))) char pull_lane_state[kPullStateBytes];
   warm_kernargs<(int)sizeof(Fused256Args)>();
   if (f.trace_start && blockIdx.x == 0 && threadIdx.x == 0) *f.trace_start = now_ticks();
   Gemm256<InT, OutT, kWithReduce, kGatherA, kBKMajor>(f.g, kPull ? (int)offsetof(Fused256Args, pull) : -1, (int)offsetof(Fused256Args, push),
                                                       (int)offsetof(Fused256Args, reduce), stage0, stage1, landing_words,
-                                                      (int)offsetof(Fused256Args, gather), pull_lane_state)
+                                                      (int)offsetof(Fused256Args, gather))
       .run(f.s, f.m, (int)blockIdx.x, (int)gridDim.x);
   __syncthreads();
   const CommArgs c = late_kernarg<CommArgs>((int)offsetof(Fused256Args, comm));
