@@ -356,15 +356,27 @@ int tccl_gemm_reducescatter(const tccl_gemm_desc* gemm, void* out, int32_t out_d
  * of the library (about 581 KiB on every GPU the process uses, for the life of the process)
  * instead of being brought in by a tccl_sync_desc.  The caller still passes the operands, the
  * gathered output and the heap view; `plan` is HOST memory and travels in the kernel
- * arguments of a small set-up kernel that also clears the calling rank's words, so every call
- * runs as launch number 1.  group_table is derived on the device from the plan's rows by the
- * rule of build_group_table (tileccl_v2/tile_group.py:214-241).
+ * arguments of a small set-up kernel that also prepares the calling rank's words for this
+ * call.  group_table is derived on the device from the plan's rows by the rule of
+ * build_group_table (tileccl_v2/tile_group.py:214-241).
+ *
+ * Launch numbers.  The library counts the calls per device and rank (host memory).  Call n of
+ * a rank stores n into its locks and brings every TileGroup counter to n * 2 *
+ * TCCL_STATIC_MAX_TILES (the set-up kernel starts the counter the group's tile count short of
+ * that), and waits for its peers' words to reach the same values: what a peer's call n - 1
+ * left behind, with the same plan or another one, never satisfies call n.  Ranks that wait on
+ * each other must therefore have made the same number of calls on their devices, as with
+ * tccl_gemm_allgather's `epoch`; a rank whose peer is a call behind waits (bounded by
+ * `spin_limit_ns`) and raises `fault`.  Words are compared as sequence numbers
+ * (tccl_word_reached), so the count may wrap.  A call recorded into a HIP graph replays with
+ * the number it was recorded with: replays of two ranks' graphs must keep the producer ahead
+ * of the consumer on the stream, as a replay cannot be told from the one before it.
+ * tccl_static_call_words returns the values call number `call` works with.
  *
  * Limits: at most TCCL_STATIC_MAX_TILES plan tiles and TCCL_STATIC_MAX_GROUPS TileGroups
  * (larger inputs are rejected with TCCL_ERR_UNSUPPORTED), groups ascending and disjoint.
- * The ranks emulated on one GPU share the array, each with its own block of words: a rank
- * that pulls finds a peer's words where that peer's own last call left them.  Calls that
- * overlap in time on one GPU race on the shared plan tables (and on their own words when
+ * The ranks emulated on one GPU share the array, each with its own block of words.  Calls
+ * that overlap in time on one GPU race on the shared plan tables (and on their own words when
  * they are calls of the same rank): order them on one stream.  The first call on a device
  * looks up the array's address (no allocation); make it before a capture begins.
  * `fault` (device int64[1] or NULL) and `spin_limit_ns` as in tccl_sync_desc.  Calls
@@ -381,6 +393,20 @@ int tccl_gemm_allgather_static(const tccl_gemm_desc* gemm, void* out, int64_t ld
                                const tccl_heap_view* heap, const tccl_static_plan* plan,
                                const tccl_transport_desc* transport, int32_t variant,
                                int64_t* fault, int64_t spin_limit_ns, void* stream);
+/* The launch number call `call` (1, 2, ...) of tccl_gemm_allgather_static stores into its locks,
+ * where it starts a TileGroup counter of `tile_count` tiles and what that counter reads once the
+ * group is complete (what a peer in its own call `call` waits for).  Host arithmetic only. */
+int tccl_static_call_words(uint32_t call, int32_t tile_count, int32_t* epoch, int32_t* counter_start,
+                           int32_t* counter_ready);
+/* Start the launch numbers of tccl_gemm_allgather_static over on the current device: every rank's
+ * next call is call 1 again, and every rank's words in the library's array are cleared by a fill
+ * kernel on `stream` (no allocation, no memset).  For ranks whose call counts have come apart (a
+ * call that gave up on its wait, a rank that was restarted): all ranks that wait on each other
+ * must reset together, with none of their calls in flight. */
+int tccl_static_reset(void* stream);
+/* The comparison every wait on a signal word uses: 1 if `word` has reached `need`, as sequence
+ * numbers (the difference modulo 2^32 is non-negative); words and thresholds may wrap. */
+int tccl_word_reached(int32_t word, int32_t need);
 
 #ifdef __cplusplus
 }

@@ -127,3 +127,49 @@ def test_xcd_remap_is_a_bijection_and_keeps_blocks(lib, total, xcds, span):
             assert (tile % block) // span == slot % xcds and (tile % block) % span == (slot % block) // xcds
         else:
             assert tile == slot
+
+
+def test_signal_words_compare_as_sequence_numbers(lib):
+    """word_reached: `word >= need` for values that have not wrapped, and across a wrap of either."""
+    reached = lib.tccl_word_reached
+    assert reached(5, 5) and reached(6, 5) and not reached(4, 5)
+    assert reached(0, 0) and not reached(0, 1)
+    top = 2**31 - 1
+    assert reached(top, top - 10) and not reached(top - 10, top)
+    assert reached(-(2**31), top)  # one past the largest int32: the word has wrapped, the threshold has not
+    assert not reached(top, -(2**31))
+    assert reached(-5, -9) and not reached(-9, -5)
+
+
+def test_static_entry_launch_numbers(lib):
+    """The bookkeeping of tccl_gemm_allgather_static: call n stores n into its locks and takes each TileGroup
+    counter from `start` to `ready` = start + tile_count; a peer in call n waits for `ready`, and nothing that an
+    earlier call left behind (with any tile count) satisfies it, nor anything call n itself writes before the
+    group is complete -- also where the 32-bit values wrap."""
+    from tileccl_amd import _lib
+
+    def words(call, tiles):
+        epoch, start, ready = C.c_int32(), C.c_int32(), C.c_int32()
+        assert lib.tccl_static_call_words(call, tiles, C.byref(epoch), C.byref(start), C.byref(ready)) == 0
+        return epoch.value, start.value, ready.value
+
+    reached = lib.tccl_word_reached
+    unit = 2 * _lib.STATIC_MAX_TILES
+    assert words(1, 7) == (1, unit - 7, unit)
+    assert words(2, 16384) == (2, 2 * unit - 16384, 2 * unit)
+    wrap = 2**32 // unit  # the call at which counter values wrap modulo 2^32
+    for call in (1, 2, 3, 1000, 65535, 65536, 65537, wrap - 1, wrap, wrap + 1, 2**31 - 2, 2**31 - 1, 2**31, 2**31 + 1, 2**32 - 1):
+        for tiles in (1, 256, 16384):
+            epoch, start, ready = words(call, tiles)
+            assert 1 <= epoch <= 2**31 - 1
+            assert (ready - start) % 2**32 == tiles
+            assert reached(ready, ready) and not reached(start, ready)
+            assert not reached((ready - 1 + 2**31) % 2**32 - 2**31, ready)  # one tile short
+            if call > 1:
+                for old_tiles in (1, 16384):
+                    old_epoch, _, old_ready = words(call - 1, old_tiles)
+                    assert not reached(old_ready, ready), (call, tiles)
+                    if old_epoch < epoch:  # (the lock value restarts at 1 after 2^31 - 1 calls)
+                        assert not reached(old_epoch, epoch)
+    for bad in ((0, 1), (1, -1), (1, 16385)):
+        assert lib.tccl_static_call_words(bad[0], bad[1], None, None, None) != 0

@@ -29,7 +29,17 @@ def static_plan(plan):
     return p
 
 
-def launch_static(lib, op, A, B, variant):
+@pytest.fixture(autouse=True)
+def fresh_launch_numbers(lib):
+    """Every test starts from call 1 on cleared words, whatever an earlier (or failed) test left behind."""
+    from tileccl_amd import _launch, _lib
+
+    _lib.check(lib.tccl_static_reset(_launch.stream_ptr()), "tccl_static_reset")
+    torch.cuda.synchronize()
+    yield
+
+
+def launch_static(lib, op, A, B, variant, spin_limit_ns=2_000_000_000):
     """`op` supplies geometry, output and heap view; none of its signal words are passed."""
     from tileccl_amd import _launch, _lib
 
@@ -40,7 +50,7 @@ def launch_static(lib, op, A, B, variant):
     plan = static_plan(op.plan)
     rc = lib.tccl_gemm_allgather_static(
         C.byref(gemm), _launch.ptr(op.out), int(op.out.stride(0)), C.byref(view), C.byref(plan), C.byref(transport),
-        _launch.VARIANTS[variant], _launch.ptr(op.words.fault), 2_000_000_000, _launch.stream_ptr(),
+        _launch.VARIANTS[variant], _launch.ptr(op.words.fault), spin_limit_ns, _launch.stream_ptr(),
     )
     _lib.check(rc, "tccl_gemm_allgather_static")
 
@@ -82,6 +92,55 @@ def test_static_words_give_the_bytes_of_caller_supplied_words(lib, variant, macr
         for rank in (0, 1):
             assert torch.equal(bits(got[rank]), bits(want[rank])), (M, rank)
         assert torch.count_nonzero(got[0][M:]).item() > 0  # the pulled block is really there
+
+
+@pytest.mark.parametrize("variant", ["s1", "s2"])
+@pytest.mark.parametrize("macro", [128, 256])
+def test_a_puller_ahead_of_its_peer_waits_and_gives_up(lib, variant, macro):
+    """Round 1 in order (push, then pull).  In round 2 the puller is issued BEFORE the pusher: the peer's words
+    still hold round 1's values, which must not satisfy round 2; the puller's bounded wait expires, it raises its
+    fault word and leaves the peer's rows of its output alone.  Nothing hangs: the wait is the kernel's own.
+    Once the pusher has caught up (and made the call the puller gave up on), the next round works again."""
+    from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+    M, N, K = 512, 384, 128
+    heaps = SymmetricHeap.create_all(64 << 20, 2)
+    try:
+        kw = dict(macro_tile=macro, tau_min_bytes=1, group_m=2)
+        puller = FusedGemmAllGather(heaps[0], M, N, torch.float16, directions="pull", **kw)
+        pusher = FusedGemmAllGather(heaps[1], M, N, torch.float16, directions="push", **kw)
+        A0, B0 = into_heap(heaps[0], seeded((M, K), 1)), into_heap(heaps[0], seeded((K, N), 2, scale=K**-0.5))
+        A1, B1 = into_heap(heaps[1], seeded((M, K), 3)), into_heap(heaps[1], seeded((K, N), 4, scale=K**-0.5))
+        for o in (puller, pusher):
+            o.out.zero_()
+        launch_static(lib, pusher, A1, B1, variant)  # round 1
+        launch_static(lib, puller, A0, B0, variant)
+        puller.check_faults()
+        pusher.check_faults()
+        first = pusher.out[M:].clone()
+        assert torch.equal(bits(puller.out[M:]), bits(first)) and torch.count_nonzero(first).item() > 0
+
+        A1.copy_(seeded((M, K), 5))  # round 2: new inputs on the pushing rank ...
+        puller.out[M:].fill_(-3.0)  # ... and a marker where its block would land
+        launch_static(lib, puller, A0, B0, variant, spin_limit_ns=200_000)  # ahead of its peer
+        torch.cuda.synchronize()
+        assert int(puller.words.fault.item()) != 0, "round 1's words satisfied round 2"
+        with pytest.raises(RuntimeError):
+            puller.check_faults()
+        assert torch.all(puller.out[M:] == -3.0), "rows were pulled although the peer had not produced them"
+        assert_gemm_close(puller.out[:M], A0.float().cpu() @ B0.float().cpu(), tight=0.004)  # its own block is there
+        puller.words.fault.zero_()
+
+        launch_static(lib, pusher, A1, B1, variant)  # the peer's round 2 (nobody waits for it any more)
+        launch_static(lib, pusher, A1, B1, variant)  # round 3, in order again
+        launch_static(lib, puller, A0, B0, variant)
+        puller.check_faults()
+        pusher.check_faults()
+        assert torch.equal(bits(puller.out[M:]), bits(pusher.out[M:]))
+        assert not torch.equal(bits(pusher.out[M:]), bits(first))  # round 3 moved the new bytes
+    finally:
+        for h in heaps:
+            h.cleanup()
 
 
 def test_static_words_reject_what_does_not_fit(lib):

@@ -297,6 +297,13 @@ def current_context() -> TileCCLContext:
     return _get_ctx()
 
 
+def install_aliases(force: bool = False) -> None:
+    """Make the reference's import names (``tileccl``, ``tileccl.ops``, ``tileccl_v2`` ...) resolve to this package."""
+    from tileccl_amd import aliases
+
+    aliases.install_aliases(force=force)
+
+
 _LAZY = {"ops": "tileccl_amd.ops", "patterns": "tileccl_amd.patterns", "v2": "tileccl_amd.v2"}
 
 
@@ -318,6 +325,7 @@ __all__ = [
     "get_world_size",
     "current_context",
     "describe_runtime_support",
+    "install_aliases",
     "TileCCLContext",
     "Tile",
     "SymmetricHeap",

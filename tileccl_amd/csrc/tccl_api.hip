@@ -710,7 +710,23 @@ static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratch)];
 
 constexpr int kMaxDevices = 64;
 StaticScratch* g_scratch_ptr[kMaxDevices];  // per device, resolved on first use
+// Calls of tccl_gemm_allgather_static so far, per device and rank (host memory: nothing is allocated).
+// Call n of a rank stores n into its locks and brings each of its TileGroup counters to n * kStaticGroupUnit,
+// so what call n - 1 left behind (or what a call with another plan left) never satisfies a peer that is in
+// its own call n: the guarantee tccl_gemm_allgather gets from the caller's growing launch numbers.
+uint32_t g_static_calls[kMaxDevices][TCCL_MAX_WORLD];
 std::mutex g_scratch_mutex;
+// What every TileGroup counter of the static words grows to per call, whatever the group's tile count (the
+// set-up kernel starts the counter that many tiles short of the next multiple): more than any group can hold.
+constexpr int32_t kStaticGroupUnit = 2 * TCCL_STATIC_MAX_TILES;
+
+void static_call_words(uint32_t call, int32_t tile_count, int32_t* epoch, int32_t* counter_start, int32_t* counter_ready) {
+  const uint32_t n = (call - 1u) % 0x7fffffffu + 1u;  // 1 .. 2^31 - 1, then 1 again: a lock value is a positive int32
+  const uint32_t ready = n * (uint32_t)kStaticGroupUnit;  // modulo 2^32, compared as sequence numbers (word_reached)
+  *epoch = (int32_t)n;
+  *counter_ready = (int32_t)ready;
+  *counter_start = (int32_t)(ready - (uint32_t)tile_count);
+}
 
 // The current device's copy of the scratch.  The first call on a device asks the runtime for
 // the symbol's address on that device (no allocation); later calls read the cached pointer.
@@ -729,12 +745,14 @@ int static_scratch(StaticScratch** out) {
   return 0;
 }
 
-// Clears rank `rank`'s words and writes the plan tables: group_table by the rule of
-// build_group_table (tileccl_v2/tile_group.py:214-241: the first group whose rows contain the
-// tile's first row, 0 if none), under the tile numbering of tile_coords.  The other ranks'
-// words are left as their own last call left them.
-__global__ void static_setup_kernel(StaticScratch* s, tccl_static_plan plan, int rank, int tile_rows, int tile_cols, int block_m,
-                                    int group_m) {
+// Prepares rank `rank`'s words for its call number `call` and writes the plan tables: group_table by the
+// rule of build_group_table (tileccl_v2/tile_group.py:214-241: the first group whose rows contain the
+// tile's first row, 0 if none), under the tile numbering of tile_coords.  A counter starts its tile count
+// short of call * kStaticGroupUnit, the table of tile counts that the kernels multiply the launch number
+// with holds kStaticGroupUnit for every group, and locks keep what the call before stored (a smaller
+// launch number).  The other ranks' words are left as their own last call left them.
+__global__ void static_setup_kernel(StaticScratch* s, tccl_static_plan plan, int rank, uint32_t call, int tile_rows, int tile_cols,
+                                    int block_m, int group_m) {
   const int total = tile_rows * tile_cols;
   StaticWords* mine = &s->words[rank];
   const int first = blockIdx.x * blockDim.x + threadIdx.x, stride = gridDim.x * blockDim.x;
@@ -744,13 +762,13 @@ __global__ void static_setup_kernel(StaticScratch* s, tccl_static_plan plan, int
     for (int g = plan.n_groups - 1; g >= 0; --g)
       if (plan.row_starts[g] <= row && row < plan.row_ends[g]) gid = g;
     s->group_table[t] = gid;
-    mine->locks[t] = 0;
   }
   for (int g = first; g < plan.n_groups; g += stride) {
     s->row_starts[g] = plan.row_starts[g];
     s->row_ends[g] = plan.row_ends[g];
-    s->tile_counts[g] = plan.tile_counts[g];
-    mine->counter[g] = 0;
+    s->tile_counts[g] = kStaticGroupUnit;
+    const uint32_t n = (call - 1u) % 0x7fffffffu + 1u;
+    mine->counter[g] = (int32_t)(n * (uint32_t)kStaticGroupUnit - (uint32_t)plan.tile_counts[g]);
     mine->barrier[g] = 0;
   }
 }
@@ -1241,13 +1259,22 @@ int tccl_gemm_allgather_static(const tccl_gemm_desc* d, void* out, int64_t ld_ou
                   plan->row_starts[g], plan->row_ends[g], plan->tile_counts[g], d->M);
   StaticScratch* sc = nullptr;
   if ((rc = static_scratch(&sc))) return rc;
-  // One small kernel clears this rank's words and (re)writes the plan tables; it is ordered
-  // before the fused launch by the stream.  Nothing is allocated and nothing is memset.
+  int device = -1;
+  TCCL_HIP(hipGetDevice(&device));
+  uint32_t call;
+  {
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    call = ++g_static_calls[device][heap->rank];
+  }
+  int32_t epoch, start, ready;
+  static_call_words(call, 0, &epoch, &start, &ready);
+  // One small kernel prepares this rank's words for this call and (re)writes the plan tables; it is
+  // ordered before the fused launch by the stream.  Nothing is allocated and nothing is memset.
   const int threads = 256;
   int blocks = (int)((tiles + threads - 1) / threads);
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(static_setup_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, sc, *plan, heap->rank, tile_rows, tile_cols,
-                     d->block_m, d->group_m);
+  hipLaunchKernelGGL(static_setup_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, sc, *plan, heap->rank, call, tile_rows,
+                     tile_cols, d->block_m, d->group_m);
   TCCL_HIP(hipGetLastError());
   tccl_sync_desc sync;
   memset(&sync, 0, sizeof sync);
@@ -1260,10 +1287,32 @@ int tccl_gemm_allgather_static(const tccl_gemm_desc* d, void* out, int64_t ld_ou
   sync.row_ends = sc->row_ends;
   sync.tile_counts = sc->tile_counts;
   sync.n_groups = plan->n_groups;
-  sync.epoch = 1;
+  sync.epoch = epoch;
   sync.fault = fault;
   sync.spin_limit_ns = spin_limit_ns;
   return allgather_impl(d, out, ld_out, heap, &sync, tr, variant, (int64_t)sizeof(StaticWords), (hipStream_t)stream);
+}
+
+int tccl_static_call_words(uint32_t call, int32_t tile_count, int32_t* epoch, int32_t* counter_start, int32_t* counter_ready) {
+  if (call == 0 || tile_count < 0 || tile_count > TCCL_STATIC_MAX_TILES || !epoch || !counter_start || !counter_ready)
+    return fail(TCCL_ERR_INVALID, "static_call_words: call numbers start at 1, tile_count within [0, %d]", TCCL_STATIC_MAX_TILES);
+  static_call_words(call, tile_count, epoch, counter_start, counter_ready);
+  return 0;
+}
+
+int tccl_word_reached(int32_t word, int32_t need) { return tccl::word_reached(word, need) ? 1 : 0; }
+
+int tccl_static_reset(void* stream) {
+  StaticScratch* sc = nullptr;
+  int rc = static_scratch(&sc);
+  if (rc) return rc;
+  int device = -1;
+  TCCL_HIP(hipGetDevice(&device));
+  {
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    for (int r = 0; r < TCCL_MAX_WORLD; ++r) g_static_calls[device][r] = 0;
+  }
+  return tccl_fill_i32((int32_t*)sc->words, (int64_t)(sizeof(sc->words) / sizeof(int32_t)), 0, stream);
 }
 
 int tccl_gemm_reducescatter(const tccl_gemm_desc* d, void* out, int32_t out_dtype, int64_t ld_out,

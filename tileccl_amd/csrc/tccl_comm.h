@@ -421,7 +421,7 @@ struct Waiter {
     bool ok = true;
     if (a.peers_resident) ranks &= 1u << a.rank;
     if (threadIdx.x == 0) {
-      const int32_t need = a.epoch * a.tile_counts[g];
+      const int32_t need = (int32_t)((uint32_t)a.epoch * (uint32_t)a.tile_counts[g]);
       for (int r = 0; r < a.world && ok; ++r)
         if ((ranks >> r) & 1u) ok = tile_wait_ge<true>(peer_words(a, a.counter, r), g, need, deadline);
       if (ok && a.trace_ready_clock) {

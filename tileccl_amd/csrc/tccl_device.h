@@ -148,14 +148,19 @@ TCCL_D int32_t tile_signal_add(int32_t* words, int i, int32_t v) {
   return __hip_atomic_fetch_add(&words[i], v, Relaxed ? __ATOMIC_RELAXED : __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// tile_wait_ge: spin until counter[i] >= threshold.  The reference reads the word with
+// Has a signal word reached the value a waiter needs?  Words only ever grow, and the comparison is the
+// one of sequence numbers (the difference, taken modulo 2^32, is non-negative): a word and a threshold
+// that have both wrapped around still compare correctly, as long as they are less than 2^31 apart.
+TCCL_HD bool word_reached(int32_t word, int32_t need) { return (int32_t)((uint32_t)word - (uint32_t)need) >= 0; }
+
+// tile_wait_ge: spin until counter[i] >= threshold (word_reached).  The reference reads the word with
 // atomic_add(0, acquire) (ipc.py:244-254); relaxed loads followed by one acquire fence
 // observe the same value without taking the line exclusive.  Bounded like tile_wait.
 template <bool Relaxed = false>
 TCCL_D bool tile_wait_ge(const int32_t* words, int i, int32_t threshold, int64_t deadline) {
   for (;;) {
     for (int s = 0; s < 32; ++s) {
-      if (__hip_atomic_load(&words[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= threshold) {
+      if (word_reached(__hip_atomic_load(&words[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), threshold)) {
         if (!Relaxed) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         return true;
       }

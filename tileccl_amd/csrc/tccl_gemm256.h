@@ -742,7 +742,7 @@ struct Gemm256 {
       st.group_units = (uint32_t)(rows < a->block_rows ? rows : a->block_rows) * a->upr;
       return;
     }
-    st.need = a->epoch * table(a->tile_counts, st.gidx);
+    st.need = (int32_t)((uint32_t)a->epoch * (uint32_t)table(a->tile_counts, st.gidx));
     st.group_units = (uint32_t)(table(a->row_ends, st.gidx) - st.row0) * a->upr;
   }
   // Byte offset, inside the peer's words, of the word this lane looks at to learn whether group
@@ -762,7 +762,7 @@ struct Gemm256 {
     return (uint32_t)(first_m * g.tile_cols + tn * height + (tm - first_m)) * 4u;
   }
   // Every lane's word has reached the threshold (one and the same word outside tile mode).
-  static TCCL_D bool all_reached(int32_t word, int32_t need) { return __builtin_amdgcn_ballot_w64(word < need) == 0ull; }
+  static TCCL_D bool all_reached(int32_t word, int32_t need) { return __builtin_amdgcn_ballot_w64(!word_reached(word, need)) == 0ull; }
   TCCL_D void pull_group_done(PullState& st, PullPtr a) const {
     st.ready_units = st.group_units;
     ++st.gidx;
@@ -1437,7 +1437,7 @@ struct Gemm256 {
               const int gi = s.group_table[tile_id];
               if (gi == waited_group) continue;
               waited_group = gi;
-              ok = tile_wait_ge<true>((const int32_t*)((const char*)ra->counter + delta), gi, ra->epoch * ra->tile_counts[gi], deadline);
+              ok = tile_wait_ge<true>((const int32_t*)((const char*)ra->counter + delta), gi, (int32_t)((uint32_t)ra->epoch * (uint32_t)ra->tile_counts[gi]), deadline);
             }
           }
       }
