@@ -342,6 +342,101 @@ class Workload:
         out = torch.empty(self.M, self.N, dtype=A.dtype, device=A.device)
         return {"kn": lambda _v: torch.matmul(A, B_kn, out=out), "nk": lambda _v: torch.matmul(A, B_nk.t(), out=out)}
 
+    def mfma_sustained(self):
+        """What the matrix pipes sustain on THIS workload's operand values with nothing else running: a loop of the
+        K loop's MFMA instruction on registers filled from A (row operands) and B (column operands), and the same
+        loop on all-zero registers (tccl_mfma_rate_probe; TFLOP/s from the difference of two loop lengths)."""
+        import torch
+
+        from tileccl_amd.v2.calibrate import mfma_sustained_tflops
+
+        kind = "f8_16x16x128" if self.in_type == "f8" else "f16_16x16x32"
+        a, b = self.A.reshape(-1), (self.B if self.b_layout == "kn" else self.B.t()).reshape(-1)
+        on_data = mfma_sustained_tflops(kind, a, b)
+        zeros = torch.zeros(1 << 22, dtype=a.dtype, device=a.device) if self.in_type != "f8" else \
+            torch.zeros(1 << 22, dtype=torch.uint8, device=a.device).view(a.dtype)
+        on_zeros = mfma_sustained_tflops(kind, zeros, zeros)
+        return {"instruction": kind, "tflops": round(on_data["tflops"], 1), "us_per_tile_step": round(on_data["us_per_step"], 4),
+                "on_zero_operands_tflops": round(on_zeros["tflops"], 1),
+                "note": "MFMAs only (operands loaded once into registers, no LDS or memory access in the loop), one workgroup of "
+                        "8 wavefronts per CU, operand registers filled from this workload's A and B; measured in this run"}
+
+    def live_pair(self, steps=100, warmup=20, wgs=128):
+        """Both ranks of the pair for real, at the same time: two launches on two streams, `wgs` workgroups each (they fit
+        side by side on the CUs), nothing preset and nothing emulated on a peer's behalf.  Each rank waits inside its
+        kernel for the words the other one is writing.  us per pair of launches, all-gather workloads only."""
+        import ctypes as C
+
+        import torch
+
+        from tileccl_amd import _launch, _lib
+        from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
+
+        if self.kind != "ag":
+            return None
+        lib = _lib.load()
+        pool = [torch.cuda.Stream() for _ in range(8)]
+        word = torch.zeros(1, dtype=torch.int32, device="cuda")
+        seen = torch.zeros(2, dtype=torch.int32, device="cuda")
+
+        def side_by_side(a, b):
+            """A one-lane kernel that waits (20 ms at most) on `a` is released by a kernel launched after it on `b`."""
+            for x, y in ((a, b), (b, a)):
+                word.zero_()
+                seen.zero_()
+                torch.cuda.synchronize()
+                lib.tccl_prim_wait_ge(_launch.ptr(word), 0, 1, 20_000_000, _launch.ptr(seen), C.c_void_p(x.cuda_stream))
+                lib.tccl_prim_signal_add(_launch.ptr(word), 0, 1, _launch.ptr(seen[1:]), C.c_void_p(y.cuda_stream))
+                torch.cuda.synchronize()
+                if int(seen[0].item()) != 1:
+                    return False
+            return True
+
+        streams = next(([a, b] for a in pool for b in pool if a is not b and side_by_side(a, b)), None)
+        if streams is None:
+            return {"us_per_pair": None, "reason": "no two streams of this process ran kernels side by side"}
+        M, N, K = self.M, self.N, self.K
+        heaps = SymmetricHeap.create_all(1 << 30, 2)
+        result = {}
+        try:
+            operands = []
+            for r, h in enumerate(heaps):
+                A, B = h.allocate_tensor((M, K), torch.float16), h.allocate_tensor((K, N), torch.float16)
+                A.copy_(seeded((M, K), 10 + r))
+                B.copy_(seeded((K, N), 15 + r, K**-0.5))
+                operands.append((A, B))
+            for directions, variants in (("push", ("s0", "s1", "s2")), ("pull", ("s1", "s2"))):
+                ops = [FusedGemmAllGather(h, M, N, torch.float16, directions=directions, block_m=self.block_m, num_gemm_wgs=wgs,
+                                          macro_tile=self.op.macro_tile, target_group_tiles=self.group_tiles,
+                                          spin_limit_ns=300_000_000) for h in heaps]
+
+                def step(variant):
+                    for rank in (1, 0):
+                        with torch.cuda.stream(streams[rank]):
+                            ops[rank](*operands[rank], variant)
+
+                for variant in variants:
+                    for _ in range(warmup):
+                        step(variant)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(steps):
+                        step(variant)
+                    torch.cuda.synchronize()
+                    result[f"{variant}_{directions}"] = round((time.perf_counter() - t0) / steps * 1e6, 2)
+                    for op in ops:
+                        op.check_faults()
+                assert torch.equal(ops[0].out[M:], ops[1].out[M:]) and torch.equal(ops[0].out[:M], ops[1].out[:M])
+        finally:
+            for h in heaps:
+                h.cleanup()
+        return {"us_per_pair": result, "workgroups_per_rank": wgs,
+                "s0_vs_s2_pull": round(result["s0_push"] / result["s2_pull"], 4),
+                "s0_vs_s2_push": round(result["s0_push"] / result["s2_push"], 4),
+                "note": "two ranks' launches at the same time on two streams, each on half of the CUs, host wall time per pair; "
+                        "S0 = GEMM then bulk push per rank; pull = each rank fetches the other's block as its TileGroups "
+                        "(S2) / tiles (S1) are published, i.e. not before the peer's K loops have produced them"}
+
     def cpu_baseline(self, iters=3):
         """The oracle's restatement of the same operation on the host cores (reported, not a target)."""
         import torch
@@ -469,6 +564,34 @@ class ChainedWorkload:
             c.heap.cleanup()
 
 
+def probe_mfma_table(repeats=3):
+    """Every instruction shape of tccl_mfma_rate_probe on all-zero and on normally distributed operands (row operands
+    N(0, 1), column operands N(0, 1/1024): the distributions of the benchmark's A and B), `repeats` measurements each."""
+    import torch
+
+    from tileccl_amd.v2.calibrate import PROBE_KINDS, mfma_sustained_tflops
+
+    g = torch.Generator().manual_seed(0)
+    n = 1 << 24
+    rows, cols = torch.randn(n, generator=g), torch.randn(n, generator=g) / 32
+    table = {}
+    for kind, (_code, _k, dtype) in PROBE_KINDS.items():
+        if dtype == torch.float8_e4m3fn:  # the fp8 recipe of the benchmark: one sigma stored as 64
+            a, b = (rows * 64).clamp(-448, 448).to(dtype).cuda(), (cols * 32 * 64).clamp(-448, 448).to(dtype).cuda()
+            zeros = torch.zeros(n, dtype=torch.uint8, device="cuda").view(dtype)
+        else:
+            a, b = rows.to(dtype).cuda(), cols.to(dtype).cuda()
+            zeros = torch.zeros(n, dtype=dtype, device="cuda")
+        peak = PEAK_TFLOPS["f8" if dtype == torch.float8_e4m3fn else "f16"]
+        for name, (x, y) in (("zeros", (zeros, zeros)), ("normal", (a, b))):
+            runs = [mfma_sustained_tflops(kind, x, y) for _ in range(repeats)]
+            best = max(runs, key=lambda r: r["tflops"])
+            table[f"{kind} {name}"] = {"tflops": round(best["tflops"], 1), "us_per_tile_step": round(best["us_per_step"], 4),
+                                       "of_published_peak": round(best["tflops"] / peak, 4),
+                                       "launch_us": [round(u, 2) for u in best["launch_us"]], "steps": best["steps"]}
+    return {"probe": "tccl_mfma_rate_probe", "workgroups": runs[0]["workgroups"], "table": table}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -489,6 +612,10 @@ def main() -> int:
                     help="B in memory: 'kn' = (K, N) row-major (the configurations' layout), 'nk' = an (N, K) tensor passed "
                          "as its .t() view (a linear layer's weight)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-live-pair", action="store_true", help="skip the two-live-ranks leg (all-gather workloads)")
+    ap.add_argument("--probe-mfma", action="store_true",
+                    help="only run the MFMA-rate probe (every instruction shape, on zeros and on normally distributed "
+                         "operands) and print its table as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: peer ranks are emulated as slices of one HBM arena, "
@@ -499,6 +626,9 @@ def main() -> int:
     from tileccl_amd.backends import get_backend
 
     _lib.load()
+    if args.probe_mfma:
+        print(json.dumps(probe_mfma_table()))
+        return 0
     props = get_backend().get_device_properties()
     if WORKLOADS[args.workload][0] == "ch":
         w = ChainedWorkload(args.workload, args.macro_tile)
@@ -575,6 +705,12 @@ def main() -> int:
             "kernel_ms": round(chosen["event_ms_mean"], 5),
         },
     }
+    if getattr(w, "mfma_sustained", None):
+        sustained = w.mfma_sustained()
+        line["roofline"]["sustained_peak"] = sustained["tflops"]  # beside `peak`, never instead of it
+        line["roofline"]["frac_of_sustained"] = round(tflops / sustained["tflops"], 4)
+        line["mfma_sustained"] = sustained
+        line["gemm_only_frac_of_sustained"] = round(line["gemm_only_tflops"] / sustained["tflops"], 4)
     if getattr(w, "calibration", None):
         line["config"]["calibration"] = w.calibration
     if args.b_layout != "kn":
@@ -604,6 +740,10 @@ def main() -> int:
             "s0_phase_gbs": round(w.exchange_bytes / (phase_ms * 1e-3) / 1e9, 1),
             "peak_gbs": PEAK_HBM_GBS,
         }
+    if not args.no_live_pair and getattr(w, "live_pair", None):
+        pair = w.live_pair()
+        if pair is not None:
+            line["live_pair"] = pair
     if not args.no_cpu:
         secs, cores = w.cpu_baseline()
         line["cpu_baseline"] = {

@@ -408,6 +408,23 @@ int tccl_static_reset(void* stream);
  * numbers (the difference modulo 2^32 is non-negative); words and thresholds may wrap. */
 int tccl_word_reached(int32_t word, int32_t need);
 
+/* ---- measurement aid: what the matrix pipes sustain by themselves ------------------------------
+ * No counterpart in the reference.  A launch shaped like the large-tile GEMM (`workgroups` x 512
+ * threads, 128 accumulator registers per lane) whose lanes load 96 operand registers once --
+ * row operands from `a_like`, column operands from `b_like`, each lane its own 16- or 32-byte
+ * units, wrapping around the buffers -- and then issue nothing but MFMAs: `steps` times the
+ * MFMAs of one K step of a 256 x 256 tile, i.e. 2 * 256 * 256 * 64 FLOP per workgroup and step
+ * for the 16-bit kinds and 2 * 256 * 256 * 128 for the fp8 kinds.  No LDS and no memory access
+ * inside the loop, so (time(steps2) - time(steps1)) / (steps2 - steps1) is the matrix pipes'
+ * own time per step on that operand data.  `sink` takes one float per thread. */
+#define TCCL_PROBE_F16_32X32X16 0
+#define TCCL_PROBE_F16_16X16X32 1
+#define TCCL_PROBE_BF16_16X16X32 2
+#define TCCL_PROBE_F8_16X16X128 3
+#define TCCL_PROBE_F8_32X32X64 4
+int tccl_mfma_rate_probe(int32_t kind, const void* a_like, int64_t a_bytes, const void* b_like,
+                         int64_t b_bytes, float* sink, int32_t steps, int32_t workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -175,6 +175,7 @@ SIGNATURES = {
     "tccl_static_call_words": (C.c_int, [C.c_uint32, _i32, _P(_i32), _P(_i32), _P(_i32)]),
     "tccl_word_reached": (C.c_int, [_i32, _i32]),
     "tccl_static_reset": (C.c_int, [_vp]),
+    "tccl_mfma_rate_probe": (C.c_int, [_i32, _vp, _i64, _vp, _i64, _vp, _i32, _i32, _vp]),
     "tccl_gemm_reducescatter": (
         C.c_int,
         [_P(GemmDesc), _vp, _i32, _i64, _P(HeapView), _P(SyncDesc), _P(TransportDesc), _i32, _i32, _vp],

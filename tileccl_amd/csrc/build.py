@@ -19,7 +19,7 @@ HERE = Path(__file__).resolve().parent
 OUT = HERE.parent / "libtileccl_hip.so"
 SOURCES = [HERE / "tccl_api.hip", HERE / "tccl_kmajor.hip"]
 HEADERS = [HERE / "tccl_device.h", HERE / "tccl_gemm.h", HERE / "tccl_gemm256.h", HERE / "tccl_kernels256.h", HERE / "tccl_comm.h",
-           HERE / "tccl_staged.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
+           HERE / "tccl_staged.h", HERE / "tccl_probe.h", HERE.parent.parent / "include" / "tileccl_hip.h"]
 
 FLAGS = [
     "--offload-arch=gfx950",

@@ -16,6 +16,7 @@
 #include "tccl_gemm.h"
 #include "tccl_gemm256.h"
 #include "tccl_kernels256.h"
+#include "tccl_probe.h"
 #include "tccl_staged.h"
 
 namespace {
@@ -1301,6 +1302,30 @@ int tccl_static_call_words(uint32_t call, int32_t tile_count, int32_t* epoch, in
 }
 
 int tccl_word_reached(int32_t word, int32_t need) { return tccl::word_reached(word, need) ? 1 : 0; }
+
+int tccl_mfma_rate_probe(int32_t kind, const void* a_like, int64_t a_bytes, const void* b_like, int64_t b_bytes, float* sink,
+                         int32_t steps, int32_t workgroups, void* stream) {
+  if (!a_like || !b_like || !sink) return fail(TCCL_ERR_INVALID, "mfma_rate_probe: NULL buffer");
+  if (a_bytes < 32 || b_bytes < 32 || a_bytes % 32 || b_bytes % 32 || a_bytes > 0x7fffffffll || b_bytes > 0x7fffffffll)
+    return fail(TCCL_ERR_INVALID, "mfma_rate_probe: operand buffers must hold a multiple of 32 bytes, below 2 GiB (got %lld, %lld)",
+                (long long)a_bytes, (long long)b_bytes);
+  if (steps < 0 || workgroups < 1) return fail(TCCL_ERR_INVALID, "mfma_rate_probe: steps=%d, workgroups=%d", steps, workgroups);
+  const dim3 grid(workgroups), block(tccl::kThreads256);
+  const char* a = (const char*)a_like;
+  const char* b = (const char*)b_like;
+  const uint32_t an = (uint32_t)a_bytes, bn = (uint32_t)b_bytes;
+  hipStream_t st = (hipStream_t)stream;
+  switch (kind) {
+    case TCCL_PROBE_F16_32X32X16: hipLaunchKernelGGL((tccl::mfma_rate_wide_kernel<_Float16>), grid, block, 0, st, a, an, b, bn, sink, steps); break;
+    case TCCL_PROBE_F16_16X16X32: hipLaunchKernelGGL((tccl::mfma_rate_kernel<_Float16>), grid, block, 0, st, a, an, b, bn, sink, steps); break;
+    case TCCL_PROBE_BF16_16X16X32: hipLaunchKernelGGL((tccl::mfma_rate_kernel<__bf16>), grid, block, 0, st, a, an, b, bn, sink, steps); break;
+    case TCCL_PROBE_F8_16X16X128: hipLaunchKernelGGL((tccl::mfma_rate_kernel<tccl::fp8e4m3>), grid, block, 0, st, a, an, b, bn, sink, steps); break;
+    case TCCL_PROBE_F8_32X32X64: hipLaunchKernelGGL((tccl::mfma_rate_wide_kernel<tccl::fp8e4m3>), grid, block, 0, st, a, an, b, bn, sink, steps); break;
+    default: return fail(TCCL_ERR_INVALID, "mfma_rate_probe: unknown kind %d", kind);
+  }
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
 
 int tccl_static_reset(void* stream) {
   StaticScratch* sc = nullptr;

@@ -133,3 +133,42 @@ def calibrate(heap: SymmetricHeap, *, gemm_shape: tuple[int, int, int] = (4096, 
     profile = CostModelCalibrator.calibrate_from_measurements(points, base, two_regime=True)
     tau = int(profile.alpha_us / profile.beta_us_per_byte) if profile.beta_us_per_byte > 0 else 0
     return Calibration(tuple(points), profile, tflops, max(tau, 1))
+
+
+# ---- what the matrix pipes sustain by themselves ------------------------------------------------------
+PROBE_KINDS = {
+    # name: (kind code of include/tileccl_hip.h, k per tile step, element type of the operands)
+    "f16_32x32x16": (0, 64, torch.float16),
+    "f16_16x16x32": (1, 64, torch.float16),
+    "bf16_16x16x32": (2, 64, torch.bfloat16),
+    "f8_16x16x128": (3, 128, torch.float8_e4m3fn),
+    "f8_32x32x64": (4, 128, torch.float8_e4m3fn),
+}
+
+
+def mfma_sustained_tflops(kind: str, a_like: torch.Tensor, b_like: torch.Tensor, *, workgroups: int | None = None,
+                          steps: tuple[int, int] = (64, 576), iters: int = 20, warmup: int = 5) -> dict:
+    """TFLOP/s of a loop of nothing but MFMAs (``tccl_mfma_rate_probe``) on operand registers filled from ``a_like``
+    (row operands) and ``b_like`` (column operands): the bound that the data and the instruction shape set for any K
+    loop, whatever feeds it.  Two loop lengths are timed and the difference is taken, so that the launch and the
+    operand loads drop out."""
+    code, step_k, dtype = PROBE_KINDS[kind]
+    if a_like.dtype != dtype or b_like.dtype != dtype:
+        raise ValueError(f"{kind} takes {dtype} operands, got {a_like.dtype} and {b_like.dtype}")
+    lib = _lib.load()
+    if workgroups is None:
+        workgroups = torch.cuda.get_device_properties(a_like.device).multi_processor_count
+    a_like, b_like = a_like.contiguous(), b_like.contiguous()
+    nbytes = [t.numel() * t.element_size() // 32 * 32 for t in (a_like, b_like)]
+    sink = torch.empty(workgroups * 512, dtype=torch.float32, device=a_like.device)
+
+    def launch(n):
+        rc = lib.tccl_mfma_rate_probe(code, _launch.ptr(a_like), nbytes[0], _launch.ptr(b_like), nbytes[1], _launch.ptr(sink), n,
+                                      workgroups, _launch.stream_ptr())
+        _lib.check(rc, "tccl_mfma_rate_probe")
+
+    us = [_per_launch_us(lambda n=n: launch(n), iters, warmup) for n in steps]
+    per_step = (us[1] - us[0]) / (steps[1] - steps[0])
+    flop = 2.0 * 256 * 256 * step_k * workgroups
+    return {"kind": kind, "us_per_step": per_step, "tflops": flop / per_step / 1e6, "launch_us": us, "steps": list(steps),
+            "workgroups": workgroups}
