@@ -178,6 +178,33 @@ def allreduce_staged(tensors):
     return [acc.to(tensors[0].dtype) for _ in tensors]
 
 
+def allreduce_staged_reference_order(tensors):
+    """What the REFERENCE's staged all-reduce leaves on each rank (_allreduce_staged_kernel,
+    /root/reference/tileccl/primitives/collectives.py:883-935): rank r starts from its own values and adds
+    the other ranks' snapshots in ascending rank order, every addition in the tensor's dtype (``_reduce_op``
+    on the loaded values, :388-400), so for three or more ranks and inexact sums the ranks may end up with
+    different bits.  This build deliberately does not reproduce that (``allreduce_staged`` above: fp32, rank
+    order, one rounding, the same bits everywhere); this function exists so that the tests can hold the
+    distance between the two: for two ranks and for exact sums they coincide, otherwise they differ by
+    rounding only."""
+    out = []
+    for r, own in enumerate(tensors):
+        acc = own.clone()
+        for p, t in enumerate(tensors):
+            if p != r:
+                acc = (acc + t).to(own.dtype)  # torch adds 16-bit CPU tensors exactly and rounds once to the dtype
+        out.append(acc)
+    return out
+
+
+def rounding_bound(tensors, additions: int):
+    """Element-wise bound on the difference between two orders / precisions of the same sum of ``tensors``:
+    ``additions`` roundings, each at most one unit in the last place of a partial sum, itself at most the sum
+    of the magnitudes."""
+    eps = {torch.float16: 2.0**-10, torch.bfloat16: 2.0**-7, torch.float32: 2.0**-23}[tensors[0].dtype]
+    return additions * eps * sum(t.float().abs() for t in tensors)
+
+
 def expected_counters(tile_counts, epoch: int = 1):
     """counter[g] after ``epoch`` launches without reset: every tile of the group signalled once each."""
     return [epoch * t for t in tile_counts]

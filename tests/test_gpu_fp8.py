@@ -163,15 +163,14 @@ def test_baseline_config_4_properties(lib, own_rows):
         A_cpu, sa = quantise((M, K), 0)
         B_cpu, sb = quantise((K, N), 1, K**-0.5)
         A, B = into_heap(heaps[0], A_cpu), into_heap(heaps[0], B_cpu)
-        g = torch.Generator(device="cuda").manual_seed(2)
-        ops[1].partial.copy_(torch.randn(M, N, generator=g, device="cuda").bfloat16())
+        peer_cpu = seeded((M, N), 2, torch.bfloat16)  # the peer's partial: bf16 N(0, 1), seeded on the CPU
 
         def gemm_ref(partial):
             rows = slice(8100, 8228)
             ref = (A_cpu[rows].float() @ B_cpu.float()) * (sa * sb)
             assert_gemm_close(partial[rows], ref, rtol=5e-2, tight=0.032)
 
-        check_full_size_config(heaps, ops, kept_ops, A, B, 8192, torch.bfloat16, gemm_ref, 100, scale_a=sa, scale_b=sb)
+        check_full_size_config(heaps, ops, kept_ops, A, B, 8192, torch.bfloat16, gemm_ref, peer_cpu, scale_a=sa, scale_b=sb)
     finally:
         for h in heaps:
             h.cleanup()

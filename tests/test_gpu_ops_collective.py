@@ -51,6 +51,41 @@ def test_gemm_allgather_column_shards(lib, variant, world, M, N, K):
             c.heap.cleanup()
 
 
+@pytest.mark.parametrize("variant", ["s1", "s2"])
+def test_gemm_reducescatter_without_the_resident_peers_promise(lib, variant):
+    """``peers_resident=False``: the launch waits for the peers' words instead of trusting that their partials are
+    there.  On a fresh context rank 0 runs first and finds no producer: its bounded wait expires and the fault word is
+    raised (with the promise it would have summed zeros silently).  Rank 1, run after it, finds rank 0's words at the
+    same launch number and its output is the sum of both partials."""
+    import tileccl_amd as tileccl
+    from tileccl_amd import ops_collective
+
+    world, M, N, K = 2, 512, 1024, 128
+    ctxs = contexts(world, 256 << 20)
+    try:
+        Ns = N // world
+        A_cpu = [seeded((M, K), 10 + r) for r in range(world)]
+        B_cpu = seeded((K, N), 1, scale=K**-0.5)
+        As = [put(c, A_cpu[r]) for r, c in enumerate(ctxs)]
+        Bs = [put(c, B_cpu) for c in ctxs]
+        Cs = [c.zeros(M, Ns, dtype=torch.float16) for c in ctxs]
+        words = [ops_collective._reduce_scatter_words(c, world, M, Ns) for c in ctxs]
+        for w in words:
+            w.spin_limit_ns = 300_000
+        tileccl.ops.gemm_reducescatter(As[0], Bs[0], Cs[0], ctx=ctxs[0], variant=variant, peers_resident=False)
+        torch.cuda.synchronize()
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            words[0].raise_if_faulted()
+        tileccl.ops.gemm_reducescatter(As[1], Bs[1], Cs[1], ctx=ctxs[1], variant=variant, peers_resident=False)
+        torch.cuda.synchronize()
+        words[1].raise_if_faulted()
+        full = sum(a.float() @ B_cpu.float() for a in A_cpu)
+        assert_gemm_close(Cs[1], full[:, Ns:], tight=0.006)
+    finally:
+        for c in ctxs:
+            c.heap.cleanup()
+
+
 @pytest.mark.parametrize("variant", ["s0", "s1", "s2"])
 @pytest.mark.parametrize("world,M,N,K", [(2, 512, 512, 256), (2, 200, 272, 72), (3, 256, 768, 128), (2, 2048, 4096, 512),
                                          (3, 768, 1536, 192)])

@@ -316,6 +316,11 @@ def test_staged_collectives_random_sizes(lib, seed):
                     ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]
                     fault = prim.allreduce_staged(ts, heaps, **how)
                     want, got = oracle.allreduce_staged(cpu), ts
+                    # The reference adds in the tensor dtype, own values first (a different order on every rank):
+                    # this build's bits (checked exactly below) stay within rounding of what it would leave.
+                    bound = oracle.rounding_bound(cpu, world - 1)
+                    for r, theirs in enumerate(oracle.allreduce_staged_reference_order(cpu)):
+                        assert torch.all((want[r].float() - theirs.float()).abs() <= bound), (tag, r)
                 elif op == "allgather":
                     cpu = [seeded((block,), 7 * call + r, dtype) for r in range(world)]
                     ts = [into_heap(h, c) for h, c in zip(heaps, cpu)]

@@ -3,7 +3,9 @@ worlds of 2 to 4 ranks, ragged M / N / K, both GEMM kernels, the three variants,
 several TileGroup sizes; a second sweep draws larger shapes (K loops of up to 32 steps, several rounds
 of large tiles).  Moved bytes and two-rank sums are bit-exact; the GEMM and the sums of
 three or more ranks (whose fp32 order is pinned elsewhere) are held to the stated tolerances.
-Combinations the library refuses (shards that are not whole tiles, ...) are skipped by their error."""
+Which combinations the library refuses is decided here, from the case's parameters (a reduce-scatter whose shards
+are not whole plan tiles): exactly those must be refused, with that message, and every other draw must run.
+Any other ValueError fails the case."""
 
 import ctypes as C
 import random
@@ -48,8 +50,24 @@ def draw(rng):
     return case
 
 
+def expected_refusal(case):
+    """The message (a regular expression) the library must refuse this case with, or None if it must run."""
+    if case["kind"] == "rs" and (case["M"] // case["world"]) % case["block_m"]:
+        return r"must split into world_size=\d+ shards of whole \d+-row plan tiles"
+    return None
+
+
 def run_case(case, seed):
-    """True: checked; None: refused by the library with a ValueError (an unsupported combination)."""
+    """True: checked; None: refused by the library exactly as expected_refusal() says it must be."""
+    refusal = expected_refusal(case)
+    if refusal is None:
+        return run_supported_case(case, seed)
+    with pytest.raises(ValueError, match=refusal):
+        run_supported_case(case, seed)
+    return None
+
+
+def run_supported_case(case, seed):
     from tileccl_amd import _launch, _lib
     from tileccl_amd.v2 import FusedGemmAllGather, FusedGemmReduceScatter, SymmetricHeap
 
@@ -58,14 +76,11 @@ def run_case(case, seed):
     try:
         A_cpu, B_cpu = seeded((M, K), seed, dtype), seeded((K, N), seed + 1, dtype, scale=K**-0.5)
         common = dict(macro_tile=case["macro"], tau_min_bytes=case["tau"], group_m=case["group_m"], block_m=case["block_m"])
-        try:
-            if case["kind"] == "ag":
-                ops = [FusedGemmAllGather(h, M, N, dtype, directions=case["directions"], **common) for h in heaps]
-            else:
-                ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=case["pdt"], out_dtype=dtype,
-                                              own_rows_in_registers=case["own"], emulate_peer=case["emul"], **common) for h in heaps]
-        except ValueError:
-            return None
+        if case["kind"] == "ag":
+            ops = [FusedGemmAllGather(h, M, N, dtype, directions=case["directions"], **common) for h in heaps]
+        else:
+            ops = [FusedGemmReduceScatter(h, M, N, partial_dtype=case["pdt"], out_dtype=dtype,
+                                          own_rows_in_registers=case["own"], emulate_peer=case["emul"], **common) for h in heaps]
         A = into_heap(heaps[0], A_cpu)
         if case["kmajor"]:
             B = heaps[0].allocate_tensor((N, K), dtype).t()
@@ -82,10 +97,7 @@ def run_case(case, seed):
                 if p:
                     o.out[p * M:(p + 1) * M].copy_(blocks[p])
             op.mark_peers_ready()
-            try:
-                op(A, B, case["variant"])
-            except ValueError:
-                return None
+            op(A, B, case["variant"])
             op.check_faults()
             torch.cuda.synchronize()
             mine = op.out[:M].clone()
@@ -103,10 +115,7 @@ def run_case(case, seed):
         for o in ops:
             o.out.zero_()
         op.mark_peers_ready()
-        try:
-            op(A, B, case["variant"])
-        except ValueError:
-            return None
+        op(A, B, case["variant"])
         op.check_faults()
         torch.cuda.synchronize()
         # The partial as a plain GEMM launch stores it (the in-register mode never writes the owned
@@ -137,7 +146,7 @@ def test_random_shapes(lib, seed):
         case = draw(rng)
         try:
             checked += 1 if run_case(case, 1000 * seed + i) else 0
-        except AssertionError as e:
+        except (AssertionError, ValueError, pytest.fail.Exception) as e:
             raise AssertionError(f"case {i} of seed {seed}: {case}: {e}") from e
     assert checked >= CASES_PER_SEED // 2  # most draws are supported combinations
 
@@ -150,7 +159,7 @@ def test_random_large_shapes(lib, seed):
         case = draw_large(rng)
         try:
             checked += 1 if run_case(case, 1000 * seed + i) else 0
-        except AssertionError as e:
+        except (AssertionError, ValueError, pytest.fail.Exception) as e:
             raise AssertionError(f"case {i} of seed {seed}: {case}: {e}") from e
     assert checked >= 20
 

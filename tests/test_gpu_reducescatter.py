@@ -146,11 +146,14 @@ def test_own_rows_kept_in_registers_give_the_same_bytes(lib, variant, world, M, 
     assert torch.equal(bits(kept_partial[shard:]), bits(plain_partial[shard:]))
 
 
-def check_full_size_config(heaps, ops, kept_ops, A, B, shard, out_dtype, gemm_ref, slab_lo, **scales):
+def check_full_size_config(heaps, ops, kept_ops, A, B, shard, out_dtype, gemm_ref, peer_cpu, **scales):
     """Shared body of the full-size reduce-scatter configurations.  `ops` store every partial;
     `kept_ops` (or None) are the same operation with the owned rows' partial kept in the
-    accumulators, which is the mode the benchmark times."""
+    accumulators, which is the mode the benchmark times.  `peer_cpu` is the peer's partial as the
+    configuration states it (seeded on the CPU); both owners' whole shards are compared with the
+    oracle's reduction of the CPU bits."""
     op = ops[0]
+    ops[1].partial.copy_(peer_cpu)
     outs = {}
     for variant in VARIANTS:
         for o in ops:
@@ -161,10 +164,10 @@ def check_full_size_config(heaps, ops, kept_ops, A, B, shard, out_dtype, gemm_re
         outs[variant] = (ops[0].out.clone(), ops[1].out.clone())
     for v in ("s1", "s2"):
         assert torch.equal(bits(outs[v][0]), bits(outs["s0"][0])) and torch.equal(bits(outs[v][1]), bits(outs["s0"][1]))
+    partials_cpu = [op.partial.cpu(), peer_cpu]  # rank 0's partial as its GEMM stored it, the peer's as seeded
     for owner in (0, 1):
-        rows = slice(owner * shard + slab_lo, owner * shard + slab_lo + 128)
-        want = (op.partial[rows].float() + ops[1].partial[rows].float()).to(out_dtype)
-        assert torch.equal(bits(outs["s2"][owner][slab_lo:slab_lo + 128]), bits(want))
+        want = oracle.reduce_rows(partials_cpu, owner, out_dtype)
+        assert torch.equal(bits(outs["s2"][owner].cpu()), bits(want)), owner
     gemm_ref(op.partial)
     assert op.signals.counter.tolist() == oracle.expected_counters(op.plan.tile_counts(), op.words.epoch)
     if kept_ops is None:
@@ -199,14 +202,13 @@ def test_baseline_config_3_properties(lib, own_rows):
         assert op.plan.n_groups == 8 and op.shard_rows == 4096
         kept_ops = [FusedGemmReduceScatter(h, M, N, own_rows_in_registers=True) for h in heaps] if own_rows else None
         A, B = into_heap(heaps[0], seeded((M, K), 0)), into_heap(heaps[0], seeded((K, N), 1, scale=K**-0.5))
-        g = torch.Generator(device="cuda").manual_seed(2)
-        ops[1].partial.normal_(generator=g)
+        peer_cpu = seeded((M, N), 2, torch.float32)  # the peer's partial: fp32 N(0, 1), seeded on the CPU
 
         def gemm_ref(partial):
             rows = slice(4000, 4128)
             assert_gemm_close(partial[rows], A[rows].float().cpu() @ B.float().cpu(), tight=1e-3)
 
-        check_full_size_config(heaps, ops, kept_ops, A, B, 4096, torch.float16, gemm_ref, 0)
+        check_full_size_config(heaps, ops, kept_ops, A, B, 4096, torch.float16, gemm_ref, peer_cpu)
     finally:
         for h in heaps:
             h.cleanup()

@@ -159,3 +159,33 @@ def test_staged_allreduce_restatement_is_pinned_without_its_own_formula():
     got = oc.allreduce_staged(three)
     assert all(t.item() == 2050.0 for t in got)
     assert ((three[0] + three[1]) + three[2]).item() == 2048.0
+
+
+def test_the_references_staged_order_known_answers():
+    """fp16 values whose sums round differently depending on the order: spacing is 2 from 2048 on, ties go to the
+    even mantissa.  Ranks hold [1, 2048, 1, 1].  The reference's order (own value first, then the others ascending,
+    every addition rounded to fp16) leaves rank 0 with ((1 + 2048 -> 2048) + 1 -> 2048) + 1 -> 2048 and rank 2 with
+    ((1 + 1) + 2048 = 2050) + 1 = 2051 -> 2052; this build's order (fp32, one rounding) gives 2051 -> 2052 everywhere."""
+    ranks = [torch.tensor([v], dtype=torch.float16) for v in (1.0, 2048.0, 1.0, 1.0)]
+    ref = oc.allreduce_staged_reference_order(ranks)
+    assert [t.item() for t in ref] == [2048.0, 2048.0, 2052.0, 2052.0]
+    ours = oc.allreduce_staged(ranks)
+    assert [t.item() for t in ours] == [2052.0] * 4
+    bound = oc.rounding_bound(ranks, 3)
+    for r in range(4):
+        assert (ours[r].float() - ref[r].float()).abs().item() <= bound.item()
+    # a dropped addend is far outside the bound
+    assert abs(2052.0 - 2048.0 - 1.0 - 1.0) <= bound.item() < 1.0 + 2048.0
+
+
+def test_the_two_staged_orders_coincide_for_two_ranks_and_for_exact_sums():
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        pair = [torch.randn(4096, generator=torch.Generator().manual_seed(3 + r)).to(dtype) for r in range(2)]
+        ref, ours = oc.allreduce_staged_reference_order(pair), oc.allreduce_staged(pair)
+        for r in range(2):
+            assert torch.equal(ref[r], ours[r])
+    g = torch.Generator().manual_seed(5)
+    exact = [torch.randint(-8, 9, (4096,), generator=g).to(torch.float16) for _ in range(5)]
+    ref, ours = oc.allreduce_staged_reference_order(exact), oc.allreduce_staged(exact)
+    for r in range(5):
+        assert torch.equal(ref[r], ours[r])

@@ -193,7 +193,7 @@ def _reduce_scatter_words(ctx, world: int, M: int, cols: int):
 
 def gemm_reducescatter(A: Any, B: Any, Cx: Any, *, ctx=None, implementation: str = "auto",
                        storage_kind: str = "symmetric", emulate_peer: bool = False, variant: str = "s2",
-                       own_rows_in_registers: bool = True) -> Any:
+                       own_rows_in_registers: bool = True, peers_resident: bool = True) -> Any:
     """``C = (sum over ranks of A_rank @ B)[:, this rank's columns]``.
 
     The partial products live in the context workspace ``"gemm_reducescatter.partial"`` of
@@ -206,8 +206,19 @@ def gemm_reducescatter(A: Any, B: Any, Cx: Any, *, ctx=None, implementation: str
     that block never leaves the accumulators as a partial, so its part of the workspace is not
     written.  ``variant`` picks the schedule (``"s0"`` bulk, ``"s1"`` tile by tile, ``"s2"``
     TileGroup).  ``emulate_peer`` (single-GPU emulation) also writes the other ranks' outputs
-    into their slices.  Ranks of this single-process build run one after another, so a launch
-    takes the peers' partials as resident and does not wait for their signals.
+    into their slices.
+
+    Precondition (``peers_resident=True``, the default): every other rank has already produced
+    its partials FOR THESE INPUTS -- its call has run to completion -- before this rank's call
+    is issued.  The launch then does not look at the peers' signal words at all and sums
+    whatever their workspaces hold; the first call on a fresh context, or a call made after
+    only some ranks have run with new inputs, returns sums over stale or zero partials (its own
+    block of the workspace is what the ranks after it read).  That is the arrangement of this
+    single-process build, whose ranks run one after another, and the reason the default is on:
+    all ranks run once to produce, then once more to reduce.  With ``peers_resident=False`` the
+    launch waits (bounded) for each peer's words to reach this launch's number and raises the
+    fault word if a producer is missing: the mode for ranks that really run side by side and
+    have made the same number of calls.
     ``implementation`` is accepted for signature parity; there is one implementation here.
     When ``M`` is not a multiple of the 128-row plan tile, one GEMM per column block and the
     bulk reduction run instead.
@@ -234,7 +245,7 @@ def gemm_reducescatter(A: Any, B: Any, Cx: Any, *, ctx=None, implementation: str
         if variant != "s0":
             words.next_epoch(variant)
         sync = words.desc(variant)
-        mode = _lib.RS_PEERS_RESIDENT | (_lib.RS_EMULATE_PEERS if emulate_peer else 0)
+        mode = (_lib.RS_PEERS_RESIDENT if peers_resident else 0) | (_lib.RS_EMULATE_PEERS if emulate_peer else 0)
         rc = lib.tccl_gemm_reducescatter(
             C.byref(gemm), _launch.ptr(Cx), _launch.dtype_code(Cx.dtype), int(Cx.stride(0)), C.byref(view), C.byref(sync),
             C.byref(transport), mode, _launch.VARIANTS[variant], stream,
