@@ -94,13 +94,17 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 template <typename InT, typename OutT>
 __global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::SignalArgs s, tccl::CommArgs c,
                                                        int num_compute, int64_t* trace_start) {
-  __shared__ __attribute__((aligned(16))) char smem[tccl::kLdsBytes];
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(1024))) char stage0[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage1[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage2[tccl::kStage128];
   if ((int)blockIdx.x < num_compute) {
     if (trace_start && blockIdx.x == 0 && threadIdx.x == 0) *trace_start = tccl::now_ticks();
-    tccl::GemmRole<InT, OutT>(g, smem).run(s, (int)blockIdx.x, num_compute);
+    tccl::GemmRole<InT, OutT>(g, stage0, stage1, stage2).run(s, (int)blockIdx.x, num_compute);
   } else {
-    tccl::comm_role(c, (int)blockIdx.x - num_compute, (int)gridDim.x - num_compute, (int*)smem);
+    tccl::comm_role(c, (int)blockIdx.x - num_compute, (int)gridDim.x - num_compute, (int*)stage0);
   }
+#endif
 }
 
 __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
@@ -186,14 +190,16 @@ int check_gemm(const tccl_gemm_desc* d) {
   return 0;
 }
 
-int gemm_span(int per_band, int group_m, int tile_cols, int xcds) {
-  // Tile ids an XCD takes from each block: whole columns of a band, as close to
-  // per_band / xcds as divides evenly.
+int gemm_span(int in_flight, int group_m, int xcds) {
+  // Tile ids an XCD takes from each block of xcds * span ids: its share of the tiles in flight, in whole
+  // columns of a band (ids run down the group_m rows of a band column, then to the next column), so that
+  // the tiles resident on an XCD at one time form a compact patch and share their operand panels in its
+  // L2.  What an XCD's L2 misses comes over the fabric, which is what bounds the 128 x 128-tile kernel:
+  // with 32 tiles in flight per XCD a patch of 8 x 4 tiles reads 12 panels, one of 8 x 2 twice over 20.
   if (xcds <= 1) return 1;
-  int cols = tile_cols / xcds;
-  if (cols < 1) cols = 1;
-  (void)per_band;
-  return cols * group_m;
+  int span = in_flight / xcds;
+  if (span >= group_m) span = span / group_m * group_m;
+  return span > 0 ? span : 1;
 }
 
 int build_gemm_args(const tccl_gemm_desc* d, const tccl_device_info& dev, tccl::GemmArgs* g) {
@@ -213,7 +219,11 @@ int build_gemm_args(const tccl_gemm_desc* d, const tccl_device_info& dev, tccl::
   g->tile_rows = (d->M + d->block_m - 1) / d->block_m;
   g->tile_cols = (d->N + d->block_n - 1) / d->block_n;
   g->xcds = dev.xcds;
-  g->span = gemm_span(d->group_m * g->tile_cols, d->group_m, g->tile_cols, dev.xcds);
+  {
+    const int total = g->tile_rows * g->tile_cols;
+    int wgs = d->num_wgs > 0 ? d->num_wgs : 2 * dev.compute_units;  // default_gemm_wgs()
+    g->span = gemm_span(wgs < total ? wgs : total, d->group_m, dev.xcds);
+  }
   g->wrap_rows = d->column_shards > 1 ? d->M / d->column_shards : 0;
   g->b_kmajor = (d->flags & TCCL_GEMM_B_KMAJOR) ? 1 : 0;
   return 0;

@@ -1,26 +1,35 @@
-// Persistent MFMA GEMM role for gfx950 (CDNA4), 16-bit inputs.
+// Persistent MFMA GEMM role for gfx950 (CDNA4), 16-bit inputs, 128 x 128 tiles.
 //
-// One workgroup = 256 threads = 4 wavefronts (2 x 2), producing 128 x 128 output
-// sub-tiles with K consumed 64 at a time.  A plan tile (block_m x block_n, multiples of
-// 128) is a small loop of such sub-tiles; when the whole plan tile is in memory the
-// workgroup publishes it (per-tile lock or per-TileGroup counter).
+// One workgroup = 256 threads = 4 wavefronts (2 x 2, wave tile 64 x 64), producing 128 x 128
+// output sub-tiles with K consumed 32 at a time through three LDS stages of 16 KiB.  A plan tile
+// (block_m x block_n, multiples of 128) is a small loop of such sub-tiles; when the whole plan
+// tile is in memory the workgroup publishes it (per-tile lock or per-TileGroup counter).
+// 48 KiB of LDS and <= 168 registers per lane let three workgroups share a CU (two that multiply
+// and one that moves data, in the fused launches), each with one wavefront per SIMD and barriers
+// of its own, so that one workgroup's waits are covered by the others' MFMAs.
 //
 // Data path of one K step
-//   global --16B/lane--> registers --> LDS --ds_read_b128--> MFMA operands
-//   LDS holds both operands "k-chunked": [k/8][row][8 values], so one 16-byte read gives
-//   a lane the 8 consecutive k it feeds to v_mfma_f32_32x32x16_{f16,bf16}.
-//   A (M x K, k-contiguous) lands in that layout directly.  B (K x N, n-contiguous) is
-//   transposed in registers on the way in: a thread owns a 4(k) x 8(n) patch, repacks it
-//   to 8 x (4 consecutive k) and writes eight 8-byte words.
-//   A k-major B (GemmArgs::b_kmajor: element (k, n) at B[n * ldb + k]) takes A's route: loaded
-//   by rows of n, it is already in the k-chunked layout.
-//   LDS is single-buffered; the next K step's global loads are issued before the MFMAs
-//   of the current one, so two workgroups per CU keep the matrix cores fed.
+//   global --buffer_load_dwordx4 ... lds--> LDS stage --ds_read--> operands of v_mfma_f32_16x16x32
+//   A stage: 128 rows x 64 B (32 k); 16-byte chunk kc of row r sits in slot kc ^ ((r >> 2) & 3), so
+//            that the 16 rows a ds_read_b128 serves in one pass cover all 64 banks.
+//   B stage: 32 k rows x 256 B (128 columns); chunk c of row k in slot c ^ 4 (k & 3) ^ 2 ((k >> 3) & 1);
+//            operands come out through ds_read_b64_tr_b16 (the transposing read: within 16 lanes,
+//            lane i supplies 4 columns of k row i / 4, lane j receives 4 k of column j), two per operand.
+//   The hardware writes lane l's 16 bytes at base + 16 l, so the swizzles are applied on the global
+//   side, by the choice of the chunk a lane fetches.  Rows >= M, columns >= N and k >= K read as
+//   zero through the buffer bounds (A chunks at k >= K are redirected past the buffer's end).
+//   A k-major B (GemmArgs::b_kmajor: element (k, n) at B[n * ldb + k]) takes A's route and layout.
 //
-// MFMA orientation: the B patch is passed as the instruction's first operand and the A
-// patch as its second, i.e. the instruction computes the transposed 32 x 32 block.  Each
-// lane then owns 4 *consecutive output columns* of one output row, which makes the
-// register->LDS->global epilogue 8/16-byte wide instead of 2-byte wide.
+// Pipeline: step t computes from stage t % 3 and issues the loads of step t + 2 into stage
+// (t + 2) % 3, which every wavefront finished reading before the barrier of step t - 1.  The
+// step's one barrier sits before its last item (of four: one 16-row block of A against the four
+// 16-column blocks of B) and waits with vmcnt(4): the four loads issued in this step may stay in
+// flight, those of the step before have landed.  Behind it the last item already fetches the
+// next step's first operands, and reloads each B operand in place once its MFMA is issued.
+//
+// MFMA orientation: the B operand is passed first, i.e. the instruction computes the transposed
+// 16 x 16 block.  Each lane then owns 4 consecutive output columns of one output row, and the
+// register -> LDS -> global epilogue moves 8 / 16 bytes per access.
 //
 // Reference semantics reproduced: C = A @ B with fp32 accumulation and one rounding to
 // the output type (tileccl/kernels/gemm.py:139-167); rows/columns past M/N are not
@@ -37,12 +46,14 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTile = 128;        // sub-tile edge
-constexpr int kBK = 64;           // K per step
-constexpr int kThreads = 256;     // threads per workgroup
-constexpr int kPlane = 130 * 16;  // bytes of one k-chunk plane: 128 rows x 16 B + 2 pad rows
-constexpr int kOperandBytes = (kBK / 8) * kPlane;  // one operand, one K step
-constexpr int kLdsBytes = 2 * kOperandBytes;       // A then B
+constexpr int kTile = 128;                        // sub-tile edge
+constexpr int kBK = 32;                           // K per step
+constexpr int kThreads = 256;                     // threads per workgroup
+constexpr int kARow128 = kBK * 2;                 // bytes of an A row in a stage
+constexpr int kAStage128 = kTile * kARow128;      // 8 192
+constexpr int kBPitch128 = kTile * 2;             // bytes of a k row of B in a stage
+constexpr int kBStage128 = kBK * kBPitch128;      // 8 192 (k-major B: 128 rows of 64 B, the same)
+constexpr int kStage128 = kAStage128 + kBStage128;  // A then B: 16 384; three such stages per workgroup
 
 enum SignalMode { kSignalNone = 0, kSignalTile = 1, kSignalGroup = 2 };
 
@@ -130,169 +141,203 @@ TCCL_D __bf16 to_out<__bf16>(float v) { return (__bf16)v; }
 template <>
 TCCL_D float to_out<float>(float v) { return v; }
 
-// 16-byte slot of row `n` inside a k-chunk plane of the B operand.  The XOR keeps both
-// the transposing writes (lanes 8 rows apart) and the MFMA reads (32 consecutive rows)
-// spread over all LDS banks.
-TCCL_D int b_slot(int n) { return n ^ (n >> 4); }
-
+#if defined(__HIP_DEVICE_COMPILE__)
 template <typename InT, typename OutT>
 struct GemmRole {
   typedef typename Mfma<InT>::Vec Vec;
+  static_assert(sizeof(InT) == 2, "16-bit inputs");
+  typedef __attribute__((address_space(3))) void LdsVoid;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 LdsQuad;
 
   const GemmArgs& g;
-  char* lds;
+  char* st0;
+  char* st1;
+  char* st2;
   const int tid, lane, wave, wm, wn;
 
-  TCCL_D GemmRole(const GemmArgs& args, char* smem)
-      : g(args), lds(smem), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
-        wm((threadIdx.x >> 6) >> 1), wn((threadIdx.x >> 6) & 1) {}
+  // The wavefront's number lives in a scalar register: the LDS addresses its loads land at derive from it.
+  TCCL_D GemmRole(const GemmArgs& args, char* s0, char* s1, char* s2)
+      : g(args), st0(s0), st1(s1), st2(s2), tid(threadIdx.x), lane(threadIdx.x & 63),
+        wave(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))), wm(wave >> 1), wn(wave & 1) {}
 
-  // ---- global -> registers ------------------------------------------------------------
-  // Loads go through buffer resources: an access past num_records returns zero, which
-  // pads rows >= M of A and rows >= K of B without branches or clamped addresses.
-  //   A: chunk c = tid + 256*i covers row (c >> 3), k-chunk (c & 7).
-  //   B: thread owns k rows 4*(tid >> 4) .. +3 and columns 8*(tid & 15) .. +7.
-  // Columns >= N of B read whatever follows in memory (still inside the buffer); they
-  // only feed output columns that are never stored.
-  struct Source {
-    __amdgpu_buffer_rsrc_t a, b;
-    uint32_t off_a[4], off_b[4];  // byte offsets of this thread's 16-byte loads, K step 0
-    uint32_t step_a, step_b;      // byte advance per K step
-  };
-
+  static TCCL_D int fresh(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+  }
   static TCCL_D uint32_t clamp_u32(int64_t v) { return v > 0xffffffffll ? 0xffffffffu : (v < 0 ? 0u : (uint32_t)v); }
 
+  // ---- global -> LDS ------------------------------------------------------------------------
+  // Per K step a wavefront fetches two 1 KiB pieces of each operand:
+  //   A piece i: rows 16 (2 wave + i) .. + 15      (lane l: row + l / 4, slot l % 4)
+  //   B piece j: k rows 4 (2 wave + j) .. + 3      (lane l: k row + l / 16, slot l % 16)
+  //   k-major B piece j: columns 16 (2 wave + j) .. + 15, as A.
+  struct Source {
+    __amdgpu_buffer_rsrc_t a, b;
+    uint32_t off_a[2], off_b[2];  // byte offsets of this lane's 16-byte loads, K step 0
+    uint32_t step_a, step_b;      // byte advance per K step
+    int k_lane;                   // first k of this lane's chunk of an A row (of a k-major B row) within a step
+  };
+
+  template <bool kBKMajor>
   TCCL_D Source make_source(int row0, int col0) const {
-    constexpr int kEsz = sizeof(InT);
     Source s;
+    const int ln = fresh(lane);
     const OperandOrigin o = operand_origin(g, row0, col0);
     const InT* A = (const InT*)g.A + (int64_t)o.a_row * g.lda;
-    const InT* B = (const InT*)g.B + (g.b_kmajor ? (int64_t)o.b_col * g.ldb : (int64_t)o.b_col);
-    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * kEsz), 0x00020000);
-    const int64_t b_elems = g.b_kmajor ? (int64_t)(o.b_cols - 1 - o.b_col) * g.ldb + g.K : (int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col);
-    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(b_elems * kEsz), 0x00020000);
+    const InT* B = (const InT*)g.B + (kBKMajor ? (int64_t)o.b_col * g.ldb : (int64_t)o.b_col);
+    s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * 2), 0x00020000);
+    const int64_t b_elems = kBKMajor ? (int64_t)(o.b_cols - 1 - o.b_col) * g.ldb + g.K : (int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col);
+    s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(b_elems * 2), 0x00020000);
+    // Bits 2 and 3 of a row's number come from the lane alone (a piece starts on a multiple of 16).
+    const int kc = (ln & 3) ^ ((ln >> 4) & 3);
+    s.k_lane = kc * 8;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      s.off_a[i] = (uint32_t)(((tid >> 3) + 32 * i) * g.lda * kEsz + (tid & 7) * 16);
-      s.off_b[i] = g.b_kmajor ? (uint32_t)(((tid >> 3) + 32 * i) * g.ldb * kEsz + (tid & 7) * 16)
-                              : (uint32_t)(((tid >> 4) * 4 + i) * g.ldb * kEsz + (tid & 15) * 16);
+    for (int i = 0; i < 2; ++i) {
+      const int row = 16 * (2 * wave + i) + (ln >> 2);
+      s.off_a[i] = (uint32_t)(row * g.lda * 2 + kc * 16);
+      if constexpr (kBKMajor) {
+        s.off_b[i] = (uint32_t)(row * g.ldb * 2 + kc * 16);
+      } else {
+        const int k = 4 * (2 * wave + i) + (ln >> 4);
+        const int c = (ln & 15) ^ (4 * (k & 3)) ^ (2 * ((k >> 3) & 1));
+        s.off_b[i] = (uint32_t)(k * g.ldb * 2 + c * 16);
+      }
     }
-    s.step_a = kBK * kEsz;
-    s.step_b = g.b_kmajor ? (uint32_t)(kBK * kEsz) : (uint32_t)(kBK * g.ldb * kEsz);
+    s.step_a = kBK * 2;
+    s.step_b = kBKMajor ? (uint32_t)(kBK * 2) : (uint32_t)(kBK * g.ldb * 2);
     return s;
   }
 
-  // `tail`: this K step reaches past K, so A chunks at k >= K must read as zero too
-  // (B rows >= K already do, being past the end of the buffer).
-  TCCL_D void load_global(const Source& s, int kt, bool tail, u32x4 (&ra)[4], u32x4 (&rb)[4]) const {
-    const uint32_t adv_a = kt * s.step_a, adv_b = kt * s.step_b;
-    const bool dead = tail && (kt * kBK + (tid & 7) * 8 >= g.K);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t off = dead ? 0xfffffff0u : s.off_a[i] + adv_a;
-      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(s.a, off, 0, 0);
-    }
-    const bool dead_b = dead && g.b_kmajor;  // row-major B: rows >= K lie past the end of the buffer
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(s.b, dead_b ? 0xfffffff0u : s.off_b[i] + adv_b, 0, 0);
+  // Piece i of both operands of K step kt, straight into `stage`.
+  template <bool kBKMajor>
+  TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
+    const bool dead = kt * kBK + s.k_lane >= g.K;
+    const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + kt * s.step_a;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + (2 * wave + i) * 1024), 16, oa, 0, 0, 0);
+    uint32_t ob = s.off_b[i] + kt * s.step_b;  // row-major B: rows >= K lie past the end of the buffer
+    if constexpr (kBKMajor) ob = dead ? 0xfffffff0u : ob;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage128 + (2 * wave + i) * 1024), 16, ob, 0, 0, 0);
   }
 
-  // ---- registers -> LDS ---------------------------------------------------------------
-  TCCL_D void store_lds(const u32x4 (&ra)[4], const u32x4 (&rb)[4]) const {
-    char* la = lds + (tid & 7) * kPlane;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4*)(la + ((tid >> 3) + 32 * i) * 16) = ra[i];
-
-    if (g.b_kmajor) {  // rb[i]: the 8 consecutive k of column (tid >> 3) + 32 * i, as the reads want them
-      char* lb = lds + kOperandBytes + (tid & 7) * kPlane;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *(u32x4*)(lb + b_slot((tid >> 3) + 32 * i) * 16) = rb[i];
-      return;
+  // ---- LDS -> MFMA operands -------------------------------------------------------------------
+  // 16 x 16 x 32 operands: lane l holds the 8 consecutive k of group l / 16 for row (column) l % 16.
+  struct Reader {
+    uint32_t a_base;   // this lane's row of A row block 0, slot applied
+    uint32_t b_base0;  // this lane's address for column block 0
+  };
+  template <bool kBKMajor>
+  TCCL_D Reader make_reader() const {
+    const int i16 = lane & 15, kg = lane >> 4;
+    Reader r;
+    r.a_base = (uint32_t)((wm * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 2) & 3)) << 4));
+    if constexpr (kBKMajor) {
+      r.b_base0 = (uint32_t)(kAStage128 + (wn * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 2) & 3)) << 4));
+    } else {
+      // Lane group kg covers k rows 8 kg .. + 7 in two transposing reads (k + 0, k + 4).
+      const int t = i16 >> 2, cq = i16 & 3;
+      const int chunk = (wn * 8 + (cq >> 1)) ^ (4 * t) ^ (2 * (kg & 1));
+      r.b_base0 = (uint32_t)(kAStage128 + (8 * kg + t) * kBPitch128 + chunk * 16 + (cq & 1) * 8);
     }
-    // rb[i] holds columns n0..n0+7 of k row i as 4 dwords (two columns each).  Column
-    // n0+j needs its four k values side by side: two dwords (k0|k1) and (k2|k3).
-    const int kg = tid >> 4;
-    char* lb = lds + kOperandBytes + (kg >> 1) * kPlane + (kg & 1) * 8;
-    const int n0 = (tid & 15) * 8;
-    const u32x4 r0 = rb[0], r1 = rb[1], r2 = rb[2], r3 = rb[3];
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      uint2 even, odd;
-      even.x = (r0[d] & 0xffffu) | (r1[d] << 16);
-      even.y = (r2[d] & 0xffffu) | (r3[d] << 16);
-      odd.x = (r0[d] >> 16) | (r1[d] & 0xffff0000u);
-      odd.y = (r2[d] >> 16) | (r3[d] & 0xffff0000u);
-      *(uint2*)(lb + b_slot(n0 + 2 * d) * 16) = even;
-      *(uint2*)(lb + b_slot(n0 + 2 * d + 1) * 16) = odd;
-    }
+    return r;
+  }
+  TCCL_D Vec load_a(const char* stage, const Reader& r, int rb) const { return *(const Vec*)(stage + r.a_base + rb * 16 * kARow128); }
+  template <bool kBKMajor>
+  TCCL_D Vec load_b(const char* stage, const Reader& r, int cb) const {
+    if constexpr (kBKMajor) return *(const Vec*)(stage + r.b_base0 + cb * 16 * kARow128);
+    // column block cb: two chunks further on (the XOR commutes with the swizzle terms)
+    const char* pb = stage + (r.b_base0 ^ (uint32_t)(32 * cb));
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)pb);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsQuad*)(pb + 4 * kBPitch128));
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(Vec, both);
   }
 
-  // ---- LDS -> MFMA, one K step -----------------------------------------------------------
-  TCCL_D void compute(f32x16 (&acc)[2][2]) const {
-    const int half = lane >> 5, l32 = lane & 31;
+  struct Frags {
+    Vec fa[4], fb[4];
+  };
+
+  // One K step: four items (A row block rb against the four B column blocks).  On entry fa[0], fa[1] and
+  // fb[0..3] hold this step's operands; items 0 and 1 fetch fa[2] and fa[3] and issue the loads of K step
+  // kt_load into `far`; the last item, behind the barrier, fetches the next step's fa[0], fa[1] from `nxt`
+  // and reloads each fb in place.
+  template <bool kBKMajor>
+  TCCL_D void k_step(const char* cur, const char* nxt, char* far, const Source& src, const Reader& rd, int kt_load,
+                     f32x4 (&acc)[4][4], Frags& f) const {
 #pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      const char* pa = lds + (2 * kk + half) * kPlane;
-      const char* pb = lds + kOperandBytes + (2 * kk + half) * kPlane;
-      Vec fa[2], fb[2];
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        fa[b] = *(const Vec*)(pa + (wm * 64 + b * 32 + l32) * 16);
-        fb[b] = *(const Vec*)(pb + b_slot(wn * 64 + b * 32 + l32) * 16);
+    for (int rb = 0; rb < 4; ++rb) {
+      if (rb == 3) {
+        // The loads of the step before (into `nxt`) have landed, this step's four may still be in flight;
+        // this wavefront's reads of `cur` are done.  The barrier is the bare instruction (__syncthreads()
+        // carries a release fence); the empty asm keeps LDS accesses from moving across it.
+        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        f.fa[0] = load_a(nxt, rd, 0);
+        f.fa[1] = load_a(nxt, rd, 1);
+      } else if (rb < 2) {
+        f.fa[rb + 2] = load_a(cur, rd, rb + 2);
+        issue_piece<kBKMajor>(far, src, kt_load, rb);
       }
 #pragma unroll
-      for (int bi = 0; bi < 2; ++bi)
-#pragma unroll
-        for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = Mfma<InT>::run(fb[bj], fa[bi], acc[bi][bj]);
+      for (int cb = 0; cb < 4; ++cb) {
+        acc[rb][cb] = Mfma<InT>::run16(f.fb[cb], f.fa[rb], acc[rb][cb]);
+        if (rb == 3) {
+          __builtin_amdgcn_sched_barrier(0);
+          f.fb[cb] = load_b<kBKMajor>(nxt, rd, cb);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
   // ---- accumulators -> LDS -> global -------------------------------------------------------
-  // Each wave stages its own 32-row slab (one bi at a time) in a private LDS window, then
-  // writes it out with 16-byte stores that are contiguous along the row.
+  // Block (rb, cb) of the wave tile: the lane holds row 16 rb + l % 16, columns 16 cb + 4 (l / 16) .. + 3.
+  // Each wavefront stages a 32-row slab (two row blocks) in its own 8 KiB window and writes it out
+  // with 16-byte stores that are contiguous along the row; a wavefront's LDS operations execute in
+  // the order issued, so nothing inside the loop waits for another wavefront.
   template <int kPolicy>
-  TCCL_D void epilogue(int row0, int col0, const f32x16 (&acc)[2][2]) const {
+  TCCL_D void epilogue(int row0, int col0, const f32x4 (&acc)[4][4]) const {
     constexpr int kEsz = sizeof(OutT);
     constexpr int kRowBytes = 64 * kEsz;       // one wave row: 64 columns
     constexpr int kChunks = kRowBytes / 16;    // 16-byte chunks per row (8 or 16)
     constexpr int kPerChunk = 16 / kEsz;       // elements per chunk
-    char* win = lds + wave * (32 * 64 * 4);    // 8 KiB window per wave (fp32 worst case)
+    char* win = (wave < 2 ? st0 : st1) + (wave & 1) * 8192;  // 8 KiB per wavefront (fp32 worst case)
     // The lane id is taken afresh: what the epilogue derives from it is invariant across tiles
     // and would otherwise be hoisted out of the tile loop and held in registers through the K loop.
-    int ln = lane;
-    asm volatile("" : "+v"(ln));
-    const int half = ln >> 5, l32 = ln & 31;
+    const int ln = fresh(lane);
+    const int i16 = ln & 15, kg = ln >> 4;
     // Stores go through a buffer resource rooted at the sub-tile so that the cache policy
     // can be chosen: plain write-back when nobody waits for the tile, device-coherent
     // write-through when a communication workgroup will read it right after the signal.
     OutT* C = (OutT*)g.C + (int64_t)row0 * g.ldc + col0;
     const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void*)C, 0, 0xffffffffu, 0x00020000);
-
+    __syncthreads();  // every wavefront has left the K loop's stages
 #pragma unroll
     for (int bi = 0; bi < 2; ++bi) {
-      __syncthreads();  // window free: K loop reads / previous slab's reads are done
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
+      for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n_local = bj * 32 + 8 * q + 4 * half;  // first of 4 consecutive columns
+        for (int cb = 0; cb < 4; ++cb) {
+          const int row = 16 * r + i16;
           OutT v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[bi][bj][4 * q + e] * g.alpha);
-          const int byte = n_local * kEsz;
-          const int chunk = (byte >> 4) ^ (l32 & 7);
-          char* p = win + l32 * kRowBytes + chunk * 16 + (byte & 15);
+          for (int e = 0; e < 4; ++e) v[e] = to_out<OutT>(acc[2 * bi + r][cb][e] * g.alpha);
+          const int byte = (16 * cb + 4 * kg) * kEsz;
+          const int chunk = (byte >> 4) ^ (row & 7);
+          char* p = win + row * kRowBytes + chunk * 16 + (byte & 15);
           if constexpr (kEsz == 2) {
             uint2 u;
             __builtin_memcpy(&u, v, 8);
             *(uint2*)p = u;
           } else {
-            uint4 u;
+            u32x4 u;
             __builtin_memcpy(&u, v, 16);
-            *(uint4*)p = u;
+            *(u32x4*)p = u;
           }
         }
-      __syncthreads();
+      asm volatile("" ::: "memory");  // staged by this wavefront itself: LDS keeps the order
 #pragma unroll
       for (int r = 0; r < (32 * kChunks) / 64; ++r) {
         const int idx = ln + 64 * r;
@@ -302,32 +347,48 @@ struct GemmRole {
         if (row0 + lrow < g.M && col0 + lcol < g.N)
           __builtin_amdgcn_raw_buffer_store_b128(v, rc, (uint32_t)((lrow * g.ldc + lcol) * kEsz), 0, kPolicy);
       }
+      asm volatile("" ::: "memory");
     }
   }
 
   // ---- one 128 x 128 sub-tile -------------------------------------------------------------------
-  template <int kPolicy>
+  template <int kPolicy, bool kBKMajor>
   TCCL_D void subtile(int row0, int col0) const {
-    f32x16 acc[2][2];
+    f32x4 acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-    u32x4 ra[4], rb[4];
-    const Source src = make_source(row0, col0);
+    const Source src = make_source<kBKMajor>(row0, col0);
+    const Reader rd = make_reader<kBKMajor>();
     const int ksteps = (g.K + kBK - 1) / kBK;
-    const bool ragged = (g.K % kBK) != 0;
-    load_global(src, 0, ragged && ksteps == 1, ra, rb);
-    for (int kt = 0; kt < ksteps; ++kt) {
-      __syncthreads();  // everyone is done reading the previous contents of LDS
-      store_lds(ra, rb);
-      __syncthreads();
-      if (kt + 1 < ksteps) load_global(src, kt + 1, ragged && kt + 2 == ksteps, ra, rb);
-      compute(acc);
+    __syncthreads();  // the previous sub-tile's epilogue has left LDS
+    issue_piece<kBKMajor>(st0, src, 0, 0);
+    issue_piece<kBKMajor>(st0, src, 0, 1);
+    issue_piece<kBKMajor>(st1, src, 1, 0);  // (past K: zeros, never consumed)
+    issue_piece<kBKMajor>(st1, src, 1, 1);
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // stage 0 has landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    Frags f;
+    f.fa[0] = load_a(st0, rd, 0);
+    f.fa[1] = load_a(st0, rd, 1);
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) f.fb[cb] = load_b<kBKMajor>(st0, rd, cb);
+    // Stages are named statically (the compiler tracks loads into LDS per array), so the loop comes in
+    // threes with an exit after every step; loads issued past K read zeros and are never consumed.
+    for (int kt = 0;; kt += 3) {
+      k_step<kBKMajor>(st0, st1, st2, src, rd, kt + 2, acc, f);
+      if (kt + 1 >= ksteps) break;
+      k_step<kBKMajor>(st1, st2, st0, src, rd, kt + 3, acc, f);
+      if (kt + 2 >= ksteps) break;
+      k_step<kBKMajor>(st2, st0, st1, src, rd, kt + 4, acc, f);
+      if (kt + 3 >= ksteps) break;
     }
+    wait_vmem();  // the look-ahead loads must not land on the epilogue's staging
     epilogue<kPolicy>(row0, col0, acc);
   }
 
@@ -341,10 +402,17 @@ struct GemmRole {
         for (int sn = 0; sn < g.block_n; sn += kTile) {
           const int row0 = tc.m * g.block_m + sm, col0 = tc.n * g.block_n + sn;
           if (row0 >= g.M || col0 >= g.N) continue;
-          if (s.mode == kSignalNone)
-            subtile<0>(row0, col0);
-          else
-            subtile<kCoherent>(row0, col0);
+          if (s.mode == kSignalNone) {
+            if (g.b_kmajor)
+              subtile<0, true>(row0, col0);
+            else
+              subtile<0, false>(row0, col0);
+          } else {
+            if (g.b_kmajor)
+              subtile<kCoherent, true>(row0, col0);
+            else
+              subtile<kCoherent, false>(row0, col0);
+          }
         }
       if (s.mode != kSignalNone) {
         // The tile was stored write-through; once every wave's stores have completed the
@@ -361,5 +429,6 @@ struct GemmRole {
     }
   }
 };
+#endif  // __HIP_DEVICE_COMPILE__
 
 }  // namespace tccl
