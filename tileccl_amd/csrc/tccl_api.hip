@@ -107,6 +107,23 @@ __global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::S
 #endif
 }
 
+// The GEMM alone on 128 x 128 tiles: no communication workgroup has to fit beside it, so it takes five
+// stages (80 KiB, two workgroups per CU): a load then has three steps and a half to arrive instead of
+// one and a half.
+template <typename InT, typename OutT>
+__global__ __launch_bounds__(256, 2) void gemm128_kernel(tccl::GemmArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(1024))) char stage0[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage1[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage2[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage3[tccl::kStage128];
+  __shared__ __attribute__((aligned(1024))) char stage4[tccl::kStage128];
+  tccl::SignalArgs s;
+  s.mode = tccl::kSignalNone;
+  tccl::GemmRole<InT, OutT, 5>(g, stage0, stage1, stage2, stage3, stage4).run(s, (int)blockIdx.x, (int)gridDim.x);
+#endif
+}
+
 __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   __shared__ int word[4];
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
@@ -308,8 +325,11 @@ int check_sync(const tccl_sync_desc* s, int variant) {
 template <typename InT, typename OutT>
 int launch_fused_t(const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c, int compute, int comm,
                    int64_t* trace_start, hipStream_t stream) {
-  hipLaunchKernelGGL((fused_kernel<InT, OutT>), dim3(compute + comm), dim3(tccl::kThreads), 0, stream, g, s, c, compute,
-                     trace_start);
+  if (comm == 0 && s.mode == tccl::kSignalNone && !trace_start)
+    hipLaunchKernelGGL((gemm128_kernel<InT, OutT>), dim3(compute), dim3(tccl::kThreads), 0, stream, g);
+  else
+    hipLaunchKernelGGL((fused_kernel<InT, OutT>), dim3(compute + comm), dim3(tccl::kThreads), 0, stream, g, s, c, compute,
+                       trace_start);
   TCCL_HIP(hipGetLastError());
   return 0;
 }

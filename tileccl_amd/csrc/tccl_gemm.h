@@ -1,12 +1,13 @@
 // Persistent MFMA GEMM role for gfx950 (CDNA4), 16-bit inputs, 128 x 128 tiles.
 //
 // One workgroup = 256 threads = 4 wavefronts (2 x 2, wave tile 64 x 64), producing 128 x 128
-// output sub-tiles with K consumed 32 at a time through three LDS stages of 16 KiB.  A plan tile
+// output sub-tiles with K consumed 32 at a time through three (or five) LDS stages of 16 KiB.  A plan tile
 // (block_m x block_n, multiples of 128) is a small loop of such sub-tiles; when the whole plan
 // tile is in memory the workgroup publishes it (per-tile lock or per-TileGroup counter).
 // 48 KiB of LDS and <= 168 registers per lane let three workgroups share a CU (two that multiply
 // and one that moves data, in the fused launches), each with one wavefront per SIMD and barriers
-// of its own, so that one workgroup's waits are covered by the others' MFMAs.
+// of its own, so that one workgroup's waits are covered by the others' MFMAs.  The GEMM alone runs
+// a five-stage form (80 KiB, two workgroups per CU).
 //
 // Data path of one K step
 //   global --buffer_load_dwordx4 ... lds--> LDS stage --ds_read--> operands of v_mfma_f32_16x16x32
@@ -20,12 +21,17 @@
 //   zero through the buffer bounds (A chunks at k >= K are redirected past the buffer's end).
 //   A k-major B (GemmArgs::b_kmajor: element (k, n) at B[n * ldb + k]) takes A's route and layout.
 //
-// Pipeline: step t computes from stage t % 3 and issues the loads of step t + 2 into stage
-// (t + 2) % 3, which every wavefront finished reading before the barrier of step t - 1.  The
-// step's one barrier sits before its last item (of four: one 16-row block of A against the four
-// 16-column blocks of B) and waits with vmcnt(4): the four loads issued in this step may stay in
-// flight, those of the step before have landed.  Behind it the last item already fetches the
-// next step's first operands, and reloads each B operand in place once its MFMA is issued.
+// Pipeline (S stages: 3 in the fused launches, 5 in the GEMM-only kernel): step t computes from stage
+// t % S and issues the loads of K step t + S - 1 into stage (t - 1) % S, which every wavefront finished
+// reading before the barrier of step t - 1; one load per item, four items per step (one 16-row block of A
+// against the four 16-column blocks of B).  The step's one barrier sits before its last item and waits
+// with vmcnt(4 (S - 2) - 1): the loads of the last S - 2 steps may stay in flight, those of K step t + 1
+// have landed.  Behind it the last item already fetches the next step's first operands, and reloads each
+// B operand in place once its MFMA is issued.
+// What bounds the tile shape: per K step a CU's address unit takes in 16 KiB (256 clocks at 64 B/clk) and
+// its LDS 16 KiB of writes and 32 KiB of reads, against 256 clocks of MFMAs: all three are level, where
+// the 256 x 256 tile has half the traffic per FLOP.  Measured at 4096 x 4096 x 1024: 41 us as it is,
+// 29 us without the global loads, 36 us without the LDS reads, 24 us with neither (and no barrier).
 //
 // MFMA orientation: the B operand is passed first, i.e. the instruction computes the transposed
 // 16 x 16 block.  Each lane then owns 4 consecutive output columns of one output row, and the
@@ -142,8 +148,9 @@ template <>
 TCCL_D float to_out<float>(float v) { return v; }
 
 #if defined(__HIP_DEVICE_COMPILE__)
-template <typename InT, typename OutT>
+template <typename InT, typename OutT, int kStages = 3>
 struct GemmRole {
+  static_assert(kStages == 3 || kStages == 5, "three stages (48 KiB: three workgroups per CU) or five (80 KiB: two)");
   typedef typename Mfma<InT>::Vec Vec;
   static_assert(sizeof(InT) == 2, "16-bit inputs");
   typedef __attribute__((address_space(3))) void LdsVoid;
@@ -155,11 +162,13 @@ struct GemmRole {
   char* st0;
   char* st1;
   char* st2;
+  char* st3;  // (five-stage form only)
+  char* st4;
   const int tid, lane, wave, wm, wn;
 
   // The wavefront's number lives in a scalar register: the LDS addresses its loads land at derive from it.
-  TCCL_D GemmRole(const GemmArgs& args, char* s0, char* s1, char* s2)
-      : g(args), st0(s0), st1(s1), st2(s2), tid(threadIdx.x), lane(threadIdx.x & 63),
+  TCCL_D GemmRole(const GemmArgs& args, char* s0, char* s1, char* s2, char* s3 = nullptr, char* s4 = nullptr)
+      : g(args), st0(s0), st1(s1), st2(s2), st3(s3), st4(s4), tid(threadIdx.x), lane(threadIdx.x & 63),
         wave(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))), wm(wave >> 1), wn(wave & 1) {}
 
   static TCCL_D int fresh(int v) {
@@ -210,15 +219,22 @@ struct GemmRole {
     return s;
   }
 
-  // Piece i of both operands of K step kt, straight into `stage`.
-  template <bool kBKMajor>
-  TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
+  // Piece i of K step kt, straight into `stage`.
+  TCCL_D void issue_a(char* stage, const Source& s, int kt, int i) const {
     const bool dead = kt * kBK + s.k_lane >= g.K;
     const uint32_t oa = dead ? 0xfffffff0u : s.off_a[i] + kt * s.step_a;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, (LdsVoid*)(stage + (2 * wave + i) * 1024), 16, oa, 0, 0, 0);
+  }
+  template <bool kBKMajor>
+  TCCL_D void issue_b(char* stage, const Source& s, int kt, int i) const {
     uint32_t ob = s.off_b[i] + kt * s.step_b;  // row-major B: rows >= K lie past the end of the buffer
-    if constexpr (kBKMajor) ob = dead ? 0xfffffff0u : ob;
+    if constexpr (kBKMajor) ob = (kt * kBK + s.k_lane >= g.K) ? 0xfffffff0u : ob;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, (LdsVoid*)(stage + kAStage128 + (2 * wave + i) * 1024), 16, ob, 0, 0, 0);
+  }
+  template <bool kBKMajor>
+  TCCL_D void issue_piece(char* stage, const Source& s, int kt, int i) const {
+    issue_a(stage, s, kt, i);
+    issue_b<kBKMajor>(stage, s, kt, i);
   }
 
   // ---- LDS -> MFMA operands -------------------------------------------------------------------
@@ -259,27 +275,34 @@ struct GemmRole {
   };
 
   // One K step: four items (A row block rb against the four B column blocks).  On entry fa[0], fa[1] and
-  // fb[0..3] hold this step's operands; items 0 and 1 fetch fa[2] and fa[3] and issue the loads of K step
-  // kt_load into `far`; the last item, behind the barrier, fetches the next step's fa[0], fa[1] from `nxt`
-  // and reloads each fb in place.
+  // fb[0..3] hold this step's operands; items 0 and 1 fetch fa[2] and fa[3]; the last item, behind the
+  // barrier, fetches the next step's fa[0], fa[1] from `nxt` and reloads each fb in place.  The four loads of
+  // K step kt_load into `far` (the stage read during the step before) go out one per item: a wavefront issues
+  // nothing else while the address unit accepts its load, and the four wavefronts reach an item together.
+  // The fourth goes out behind the barrier, so at the barrier the loads that may still be in flight are
+  // those of the kStages - 2 steps before, less that one.
+  static constexpr int kInFlight = 4 * (kStages - 2) - 1;
   template <bool kBKMajor>
   TCCL_D void k_step(const char* cur, const char* nxt, char* far, const Source& src, const Reader& rd, int kt_load,
                      f32x4 (&acc)[4][4], Frags& f) const {
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
       if (rb == 3) {
-        // The loads of the step before (into `nxt`) have landed, this step's four may still be in flight;
-        // this wavefront's reads of `cur` are done.  The barrier is the bare instruction (__syncthreads()
-        // carries a release fence); the empty asm keeps LDS accesses from moving across it.
-        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        // The loads of K step t + 1 (into `nxt`) have landed; this wavefront's reads of `cur` are done.
+        // The barrier is the bare instruction (__syncthreads() carries a release fence); the empty asm
+        // keeps LDS accesses from moving across it.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kInFlight) : "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         f.fa[0] = load_a(nxt, rd, 0);
         f.fa[1] = load_a(nxt, rd, 1);
       } else if (rb < 2) {
         f.fa[rb + 2] = load_a(cur, rd, rb + 2);
-        issue_piece<kBKMajor>(far, src, kt_load, rb);
       }
+      if (rb & 1)
+        issue_b<kBKMajor>(far, src, kt_load, rb >> 1);
+      else
+        issue_a(far, src, kt_load, rb >> 1);
 #pragma unroll
       for (int cb = 0; cb < 4; ++cb) {
         acc[rb][cb] = Mfma<InT>::run16(f.fb[cb], f.fa[rb], acc[rb][cb]);
@@ -366,11 +389,19 @@ struct GemmRole {
     const Reader rd = make_reader<kBKMajor>();
     const int ksteps = (g.K + kBK - 1) / kBK;
     __syncthreads();  // the previous sub-tile's epilogue has left LDS
+    // K steps 0 .. kStages - 2 go out up front (past K: zeros, never consumed); the order within a step is
+    // the one k_step() issues in (A 0, B 0, A 1, B 1).
     issue_piece<kBKMajor>(st0, src, 0, 0);
     issue_piece<kBKMajor>(st0, src, 0, 1);
-    issue_piece<kBKMajor>(st1, src, 1, 0);  // (past K: zeros, never consumed)
+    issue_piece<kBKMajor>(st1, src, 1, 0);
     issue_piece<kBKMajor>(st1, src, 1, 1);
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // stage 0 has landed
+    if constexpr (kStages == 5) {
+      issue_piece<kBKMajor>(st2, src, 2, 0);
+      issue_piece<kBKMajor>(st2, src, 2, 1);
+      issue_piece<kBKMajor>(st3, src, 3, 0);
+      issue_piece<kBKMajor>(st3, src, 3, 1);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (kStages - 2)) : "memory");  // stage 0 has landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     Frags f;
@@ -378,15 +409,31 @@ struct GemmRole {
     f.fa[1] = load_a(st0, rd, 1);
 #pragma unroll
     for (int cb = 0; cb < 4; ++cb) f.fb[cb] = load_b<kBKMajor>(st0, rd, cb);
-    // Stages are named statically (the compiler tracks loads into LDS per array), so the loop comes in
-    // threes with an exit after every step; loads issued past K read zeros and are never consumed.
-    for (int kt = 0;; kt += 3) {
-      k_step<kBKMajor>(st0, st1, st2, src, rd, kt + 2, acc, f);
-      if (kt + 1 >= ksteps) break;
-      k_step<kBKMajor>(st1, st2, st0, src, rd, kt + 3, acc, f);
-      if (kt + 2 >= ksteps) break;
-      k_step<kBKMajor>(st2, st0, st1, src, rd, kt + 4, acc, f);
-      if (kt + 3 >= ksteps) break;
+    // Step t computes from stage t % kStages, fetches its last operands from the next one and loads K step
+    // t + kStages - 1 into the one before.  Stages are named statically (the compiler tracks loads into LDS
+    // per array), so the loop comes in rounds of kStages steps with an exit after every step.
+    if constexpr (kStages == 3) {
+      for (int kt = 0;; kt += 3) {
+        k_step<kBKMajor>(st0, st1, st2, src, rd, kt + 2, acc, f);
+        if (kt + 1 >= ksteps) break;
+        k_step<kBKMajor>(st1, st2, st0, src, rd, kt + 3, acc, f);
+        if (kt + 2 >= ksteps) break;
+        k_step<kBKMajor>(st2, st0, st1, src, rd, kt + 4, acc, f);
+        if (kt + 3 >= ksteps) break;
+      }
+    } else {
+      for (int kt = 0;; kt += 5) {
+        k_step<kBKMajor>(st0, st1, st4, src, rd, kt + 4, acc, f);
+        if (kt + 1 >= ksteps) break;
+        k_step<kBKMajor>(st1, st2, st0, src, rd, kt + 5, acc, f);
+        if (kt + 2 >= ksteps) break;
+        k_step<kBKMajor>(st2, st3, st1, src, rd, kt + 6, acc, f);
+        if (kt + 3 >= ksteps) break;
+        k_step<kBKMajor>(st3, st4, st2, src, rd, kt + 7, acc, f);
+        if (kt + 4 >= ksteps) break;
+        k_step<kBKMajor>(st4, st0, st3, src, rd, kt + 8, acc, f);
+        if (kt + 5 >= ksteps) break;
+      }
     }
     wait_vmem();  // the look-ahead loads must not land on the epilogue's staging
     epilogue<kPolicy>(row0, col0, acc);
