@@ -11,8 +11,10 @@
 //
 // Data path of one K step
 //   global --buffer_load_dwordx4 ... lds--> LDS stage --ds_read--> operands of v_mfma_f32_16x16x32
-//   A stage: 128 rows x 64 B (32 k); 16-byte chunk kc of row r sits in slot kc ^ ((r >> 2) & 3), so
-//            that the 16 rows a ds_read_b128 serves in one pass cover all 64 banks.
+//   A stage: 128 rows x 64 B (32 k); 16-byte chunk kc of row r sits in slot kc ^ ((r >> 1) & 3).  (Measured
+//            with the LDS saturated by eight wavefronts: a ds_read_b128 of rows l % 16, chunk l / 16 takes
+//            1.78 times as long with ((r >> 2) & 3) or with no swizzle at all, and no longer than a
+//            conflict-free read with this term.)
 //   B stage: 32 k rows x 256 B (128 columns); chunk c of row k in slot c ^ 4 (k & 3) ^ 2 ((k >> 3) & 1);
 //            operands come out through ds_read_b64_tr_b16 (the transposing read: within 16 lanes,
 //            lane i supplies 4 columns of k row i / 4, lane j receives 4 k of column j), two per operand.
@@ -199,8 +201,8 @@ struct GemmRole {
     s.a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, clamp_u32(((int64_t)(o.a_rows - 1 - o.a_row) * g.lda + g.K) * 2), 0x00020000);
     const int64_t b_elems = kBKMajor ? (int64_t)(o.b_cols - 1 - o.b_col) * g.ldb + g.K : (int64_t)(g.K - 1) * g.ldb + (o.b_cols - o.b_col);
     s.b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, clamp_u32(b_elems * 2), 0x00020000);
-    // Bits 2 and 3 of a row's number come from the lane alone (a piece starts on a multiple of 16).
-    const int kc = (ln & 3) ^ ((ln >> 4) & 3);
+    // Bits 1 and 2 of a row's number come from the lane alone (a piece starts on a multiple of 16).
+    const int kc = (ln & 3) ^ ((ln >> 3) & 3);
     s.k_lane = kc * 8;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -247,9 +249,9 @@ struct GemmRole {
   TCCL_D Reader make_reader() const {
     const int i16 = lane & 15, kg = lane >> 4;
     Reader r;
-    r.a_base = (uint32_t)((wm * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 2) & 3)) << 4));
+    r.a_base = (uint32_t)((wm * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 1) & 3)) << 4));
     if constexpr (kBKMajor) {
-      r.b_base0 = (uint32_t)(kAStage128 + (wn * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 2) & 3)) << 4));
+      r.b_base0 = (uint32_t)(kAStage128 + (wn * 64 + i16) * kARow128 + ((kg ^ ((i16 >> 1) & 3)) << 4));
     } else {
       // Lane group kg covers k rows 8 kg .. + 7 in two transposing reads (k + 0, k + 4).
       const int t = i16 >> 2, cq = i16 & 3;
