@@ -302,6 +302,10 @@ int tccl_allreduce_staged(void* tensor, int32_t dtype, int64_t numel, void* stag
  * variant S2: one launch; GEMM workgroups add to counter[group_table[tile]];
  *             communication workgroups wait per TileGroup and move copy_elems-sized
  *             tasks (reference README.md:66-84; contract in the tileccl_v2 modules).
+ * In S1 and S2 the pushes of an all-scatter / all-gather leave from the GEMM's epilogue (the tile goes to
+ * the peers' slices from the registers it is stored from, ahead of its signal); the communication
+ * workgroups carry the pulls and the reductions, and barrier[g] counts those tasks only.  A launch with
+ * trace pointers keeps the pushes as tasks of the communication workgroups.
  * With the 256 x 256 GEMM tile (gemm->macro_tile) S1 and S2 are still one launch, but a
  * workgroup fills its CU, so the communication is done by the GEMM workgroups themselves:
  * pushes leave from the epilogue, all-gather pulls run inside the K loops (gated on the

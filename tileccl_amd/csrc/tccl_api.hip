@@ -92,7 +92,7 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // data.  Three waves per SIMD (two GEMM workgroups plus one communication workgroup per
 // CU) bounds the register budget.
 template <typename InT, typename OutT>
-__global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::SignalArgs s, tccl::CommArgs c,
+__global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::SignalArgs s, tccl::CommArgs c, tccl::PushArgs push,
                                                        int num_compute, int64_t* trace_start) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(1024))) char stage0[tccl::kStage128];
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256, 3) void fused_kernel(tccl::GemmArgs g, tccl::S
   __shared__ __attribute__((aligned(1024))) char stage2[tccl::kStage128];
   if ((int)blockIdx.x < num_compute) {
     if (trace_start && blockIdx.x == 0 && threadIdx.x == 0) *trace_start = tccl::now_ticks();
-    tccl::GemmRole<InT, OutT>(g, stage0, stage1, stage2).run(s, (int)blockIdx.x, num_compute);
+    tccl::GemmRole<InT, OutT>(g, push, stage0, stage1, stage2).run(s, (int)blockIdx.x, num_compute);
   } else {
     tccl::comm_role(c, (int)blockIdx.x - num_compute, (int)gridDim.x - num_compute, (int*)stage0);
   }
@@ -120,7 +120,9 @@ __global__ __launch_bounds__(256, 2) void gemm128_kernel(tccl::GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) char stage4[tccl::kStage128];
   tccl::SignalArgs s;
   s.mode = tccl::kSignalNone;
-  tccl::GemmRole<InT, OutT, 5>(g, stage0, stage1, stage2, stage3, stage4).run(s, (int)blockIdx.x, (int)gridDim.x);
+  tccl::PushArgs push;
+  push.world = 0;
+  tccl::GemmRole<InT, OutT, 5>(g, push, stage0, stage1, stage2, stage3, stage4).run(s, (int)blockIdx.x, (int)gridDim.x);
 #endif
 }
 
@@ -323,23 +325,26 @@ int check_sync(const tccl_sync_desc* s, int variant) {
 // Launchers
 // ------------------------------------------------------------------------------------------
 template <typename InT, typename OutT>
-int launch_fused_t(const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c, int compute, int comm,
-                   int64_t* trace_start, hipStream_t stream) {
+int launch_fused_t(const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c, const tccl::PushArgs& push,
+                   int compute, int comm, int64_t* trace_start, hipStream_t stream) {
   if (comm == 0 && s.mode == tccl::kSignalNone && !trace_start)
     hipLaunchKernelGGL((gemm128_kernel<InT, OutT>), dim3(compute), dim3(tccl::kThreads), 0, stream, g);
   else
-    hipLaunchKernelGGL((fused_kernel<InT, OutT>), dim3(compute + comm), dim3(tccl::kThreads), 0, stream, g, s, c, compute,
+    hipLaunchKernelGGL((fused_kernel<InT, OutT>), dim3(compute + comm), dim3(tccl::kThreads), 0, stream, g, s, c, push, compute,
                        trace_start);
   TCCL_HIP(hipGetLastError());
   return 0;
 }
 
 int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tccl::SignalArgs& s, const tccl::CommArgs& c,
-                 int compute, int comm, int64_t* trace_start, hipStream_t stream) {
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_fused_t<_Float16, _Float16>(g, s, c, compute, comm, trace_start, stream);
-  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused_t<_Float16, float>(g, s, c, compute, comm, trace_start, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused_t<__bf16, __bf16>(g, s, c, compute, comm, trace_start, stream);
-  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused_t<__bf16, float>(g, s, c, compute, comm, trace_start, stream);
+                 int compute, int comm, int64_t* trace_start, hipStream_t stream, const tccl::PushArgs* push_args = nullptr) {
+  tccl::PushArgs push;
+  memset(&push, 0, sizeof push);
+  if (push_args) push = *push_args;
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F16) return launch_fused_t<_Float16, _Float16>(g, s, c, push, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_F16 && out_dtype == TCCL_F32) return launch_fused_t<_Float16, float>(g, s, c, push, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_BF16) return launch_fused_t<__bf16, __bf16>(g, s, c, push, compute, comm, trace_start, stream);
+  if (in_dtype == TCCL_BF16 && out_dtype == TCCL_F32) return launch_fused_t<__bf16, float>(g, s, c, push, compute, comm, trace_start, stream);
   return fail(TCCL_ERR_UNSUPPORTED, "gemm: no kernel for in_dtype=%d, out_dtype=%d", in_dtype, out_dtype);
 }
 
@@ -686,7 +691,17 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     s.group_table = sync->group_table;
     c.granularity = tccl::kPerGroup;
   }
-  return launch_fused(d->in_dtype, d->out_dtype, g, s, c, compute, comm, trace_start, stream);
+  // Pushes leave from the GEMM's epilogue (the tile goes to the peers from the registers it is stored from and
+  // is never read back); what remains for the communication workgroups are pulls and reductions.  A traced
+  // launch keeps the pushes in the communication role, whose tasks carry the per-group clock stamps.
+  tccl::PushArgs push;
+  memset(&push, 0, sizeof push);
+  const bool traced = sync->trace_start_clock || sync->trace_ready_clock || sync->trace_done_clock;
+  if (!traced && build_push(c, g, &push)) {
+    c.directions &= ~tccl::kDirPush;
+    if (c.op != tccl::kOpReduceScatter && !(c.directions & tccl::kDirPull)) comm = 0;
+  }
+  return launch_fused(d->in_dtype, d->out_dtype, g, s, c, compute, comm, trace_start, stream, &push);
 }
 
 

@@ -121,6 +121,19 @@ struct SignalArgs {
   int64_t* trace_ready_clock;
 };
 
+// all-scatter / all-gather folded into the GEMM: the tile goes out from the staging LDS it
+// already sits in, instead of being written, signalled, re-read and copied by a second party
+// (reference: the per-tile scatter of patterns/_helpers.py:86-199, tile_allgather of
+// primitives/collectives.py:613-663).
+struct PushArgs {
+  int world;           // ranks; every rank but `rank` is a target.  0: the epilogue writes C only
+  int rank;
+  int col_lo, col_hi;  // columns of C that travel
+  int col_shift;       // target column = C column + col_shift
+  int64_t ld;          // target pitch in elements
+  const int64_t* heap_bases;  // C's address inside target q is C + heap_bases[q] - heap_bases[rank]
+};
+
 template <typename T>
 struct Mfma;
 template <>
@@ -161,6 +174,7 @@ struct GemmRole {
   typedef __attribute__((address_space(3))) s16x4 LdsQuad;
 
   const GemmArgs& g;
+  const PushArgs& push;  // world == 0: nothing leaves from the epilogue
   char* st0;
   char* st1;
   char* st2;
@@ -169,8 +183,9 @@ struct GemmRole {
   const int tid, lane, wave, wm, wn;
 
   // The wavefront's number lives in a scalar register: the LDS addresses its loads land at derive from it.
-  TCCL_D GemmRole(const GemmArgs& args, char* s0, char* s1, char* s2, char* s3 = nullptr, char* s4 = nullptr)
-      : g(args), st0(s0), st1(s1), st2(s2), st3(s3), st4(s4), tid(threadIdx.x), lane(threadIdx.x & 63),
+  TCCL_D GemmRole(const GemmArgs& args, const PushArgs& push_args, char* s0, char* s1, char* s2, char* s3 = nullptr,
+                  char* s4 = nullptr)
+      : g(args), push(push_args), st0(s0), st1(s1), st2(s2), st3(s3), st4(s4), tid(threadIdx.x), lane(threadIdx.x & 63),
         wave(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))), wm(wave >> 1), wn(wave & 1) {}
 
   static TCCL_D int fresh(int v) {
@@ -363,14 +378,36 @@ struct GemmRole {
           }
         }
       asm volatile("" ::: "memory");  // staged by this wavefront itself: LDS keeps the order
+      constexpr int kRounds = (32 * kChunks) / 64;
+      u32x4 v[kRounds];
+      int lrow[kRounds], lcol[kRounds];
+      bool live[kRounds];
 #pragma unroll
-      for (int r = 0; r < (32 * kChunks) / 64; ++r) {
+      for (int r = 0; r < kRounds; ++r) {
         const int idx = ln + 64 * r;
         const int row = idx / kChunks, chunk = idx % kChunks;
-        const u32x4 v = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
-        const int lrow = wm * 64 + bi * 32 + row, lcol = wn * 64 + chunk * kPerChunk;
-        if (row0 + lrow < g.M && col0 + lcol < g.N)
-          __builtin_amdgcn_raw_buffer_store_b128(v, rc, (uint32_t)((lrow * g.ldc + lcol) * kEsz), 0, kPolicy);
+        v[r] = *(const u32x4*)(win + row * kRowBytes + ((chunk ^ (row & 7)) * 16));
+        lrow[r] = wm * 64 + bi * 32 + row;
+        lcol[r] = wn * 64 + chunk * kPerChunk;
+        live[r] = row0 + lrow[r] < g.M && col0 + lcol[r] < g.N;
+        if (live[r]) __builtin_amdgcn_raw_buffer_store_b128(v[r], rc, (uint32_t)((lrow[r] * g.ldc + lcol[r]) * kEsz), 0, kPolicy);
+      }
+      // Fused push: the same chunks go to every peer's slice from the registers they sit in; the tile is
+      // never read back.  The signal that follows the tile's last store covers these stores as well.
+      for (int t = 0; t < push.world; ++t) {
+        if (t == push.rank) continue;
+        const int64_t push_ld = push.ld;
+        const int col_lo = push.col_lo, col_hi = push.col_hi;
+        typedef const __attribute__((address_space(4))) int64_t* Bases;
+        const int64_t delta = ((Bases)push.heap_bases)[t] - ((Bases)push.heap_bases)[push.rank];
+        char* base = (char*)g.C + delta + ((int64_t)row0 * push_ld + col0 + push.col_shift) * kEsz;
+        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xffffffffu, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+          const int col = col0 + lcol[r];
+          if (live[r] && col >= col_lo && col < col_hi)
+            __builtin_amdgcn_raw_buffer_store_b128(v[r], rt, (uint32_t)((lrow[r] * push_ld + lcol[r]) * kEsz), 0, kCoherent);
+        }
       }
       asm volatile("" ::: "memory");
     }

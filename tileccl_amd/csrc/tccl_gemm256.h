@@ -89,19 +89,6 @@ struct Macro {
 
 // Where the epilogue sends a finished tile besides C: the same rows of every listed target,
 // columns [col_lo, col_hi) of C landing at column + col_shift.  This is the push half of an
-// all-scatter / all-gather folded into the GEMM: the tile goes out from the staging LDS it
-// already sits in, instead of being written, signalled, re-read and copied by a second party
-// (reference: the per-tile scatter of patterns/_helpers.py:86-199, tile_allgather of
-// primitives/collectives.py:613-663).
-struct PushArgs {
-  int world;           // ranks; every rank but `rank` is a target.  0: the epilogue writes C only
-  int rank;
-  int col_lo, col_hi;  // columns of C that travel
-  int col_shift;       // target column = C column + col_shift
-  int64_t ld;          // target pitch in elements
-  const int64_t* heap_bases;  // C's address inside target q is C + heap_bases[q] - heap_bases[rank]
-};
-
 // Reduce-scatter carried out tile by tile.  Once a macro tile's partial is stored and
 // published, the workgroup waits for the other ranks' partials of the same tile, streams the
 // tile back, adds in fp32 -- the owner's addend
