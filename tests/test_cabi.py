@@ -111,7 +111,8 @@ def test_device_tile_order_equals_the_reference_swizzle(lib, tile_rows, tile_col
     assert lib.tccl_tile_coords(tile_rows * tile_cols, tile_rows, tile_cols, group_m, C.byref(tm), C.byref(tn)) != 0
 
 
-@pytest.mark.parametrize("total,xcds,span", [(1024, 8, 32), (1000, 8, 32), (16, 8, 8), (2048, 8, 32), (513, 8, 4), (64, 1, 1), (4096, 8, 64)])
+@pytest.mark.parametrize("total,xcds,span", [(1024, 8, 32), (1000, 8, 32), (16, 8, 8), (2048, 8, 32), (513, 8, 4), (64, 1, 1), (4096, 8, 64),
+                                             (1024, 8, 64), (256, 8, 32), (576, 8, 64), (100, 8, 12), (7, 8, 1)])
 def test_xcd_remap_is_a_bijection_and_keeps_blocks(lib, total, xcds, span):
     out = C.c_int32()
     ids = []

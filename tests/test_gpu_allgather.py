@@ -292,3 +292,32 @@ def test_baseline_config_2_with_the_group_size_chosen_by_the_cost_model(lib, blo
     finally:
         for h in heaps:
             h.cleanup()
+
+
+@pytest.mark.parametrize("macro", MACRO)
+def test_fused_launches_give_the_bulk_variant_bits_for_every_k_loop_length(lib, macro):
+    """S0 runs the GEMM alone (on the 128 tile: five LDS stages), S1 / S2 the fused tile loop (three stages, pushes
+    from the epilogue): the sums are formed in the same order, so the gathered bytes are the same, for every length
+    of the K loop."""
+    M, N = 256, 384
+    for K in (8, 40, 64, 96, 136, 160, 200, 224, 296, 320):
+        heaps, ops = make(2, M, N, macro_tile=macro, heap_bytes=64 << 20)
+        try:
+            op = ops[0]
+            A, B = into_heap(heaps[0], seeded((M, K), 20 + K)), into_heap(heaps[0], seeded((K, N), 21 + K, scale=K**-0.5))
+            blocks = fill_peer_blocks(ops, M, N, torch.float16)
+            got = {}
+            for variant in VARIANTS:
+                op.out[:M].zero_()
+                op.peer_out(1)[:M].zero_()
+                op.mark_peers_ready()
+                op(A, B, variant)
+                op.check_faults()
+                got[variant] = (bits(op.out).clone(), bits(op.peer_out(1)).clone())
+            for variant in ("s1", "s2"):
+                assert torch.equal(got[variant][0], got["s0"][0]), (K, variant)
+                assert torch.equal(got[variant][1], got["s0"][1]), (K, variant)
+            assert torch.equal(got["s0"][0][M:].cpu(), bits(blocks[1]))
+        finally:
+            for h in heaps:
+                h.cleanup()

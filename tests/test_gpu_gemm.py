@@ -157,3 +157,20 @@ def test_unsupported_layouts_fail_loudly(lib):
     with pytest.raises(ValueError, match="no kernel for in_dtype"):
         d = _launch.gemm_desc(A, B, torch.empty(128, 128, dtype=torch.bfloat16, device="cuda"))
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+
+
+@pytest.mark.parametrize("macro", MACRO)
+def test_every_length_of_the_k_loop(lib, macro):
+    """K from one chunk to a dozen steps, ragged tails included: the staged K loops (three or five stages of 32 k on
+    the 128 tile, two of 64 k on the large tile) leave through each of their exits, and the look-ahead loads past K
+    never reach a sum."""
+    for K in (8, 24, 32, 40, 64, 96, 104, 128, 136, 160, 168, 192, 200, 224, 256, 296, 320, 352, 384, 776):
+        A, B = seeded((256, K), 10 + K), seeded((K, 136), 11 + K, scale=K**-0.5)
+        got = run_gemm(lib, A, B, torch.float16, macro_tile=macro)
+        assert_gemm_close(got, A.float() @ B.float(), tight=0.004)
+        # integer-valued operands: every partial sum is exact, so the result is exact whatever the step structure
+        g = torch.Generator().manual_seed(K)
+        Ai = torch.randint(-2, 3, (130, K), generator=g).half()
+        Bi = torch.randint(-2, 3, (K, 72), generator=g).half()
+        want = (Ai.float() @ Bi.float()).half()
+        assert torch.equal(run_gemm(lib, Ai, Bi, torch.float16, macro_tile=macro).cpu(), want), K
