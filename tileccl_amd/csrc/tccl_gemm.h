@@ -416,13 +416,21 @@ struct GemmRole {
   // ---- one 128 x 128 sub-tile -------------------------------------------------------------------
   template <int kPolicy, bool kBKMajor>
   TCCL_D void subtile(int row0, int col0) const {
-    f32x4 acc[4][4];
+    f32x4 acc[4][4];  // cleared two registers per instruction
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j) {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+        f64x2 z;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 2; ++e) {
+          double d;
+          asm volatile("v_mov_b64 %0, 0" : "=v"(d));
+          z[e] = d;
+        }
+        acc[i][j] = __builtin_bit_cast(f32x4, z);
+      }
 
     const Source src = make_source<kBKMajor>(row0, col0);
     const Reader rd = make_reader<kBKMajor>();

@@ -1278,13 +1278,23 @@ struct Gemm256 {
     // accumulators flow through one straight loop body.  An odd step count is rounded up: the
     // extra step (like the final look-ahead load) lies wholly past K and reads zeros.
     const int ksteps = ((g.K + kStepK - 1) / kStepK + 1) & ~1;
+    // The accumulators are cleared two registers per instruction (64-bit moves): 128 single moves per
+    // wavefront, two wavefronts per SIMD, were half a microsecond of a tile's start.
     f32x16 acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j) {
+        typedef double f64x8 __attribute__((ext_vector_type(8)));
+        f64x8 z;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 8; ++e) {
+          double d;
+          asm volatile("v_mov_b64 %0, 0" : "=v"(d));
+          z[e] = d;
+        }
+        acc[i][j] = __builtin_bit_cast(f32x16, z);
+      }
     const Reader rd = make_reader();
     wait_vmem();  // the first operands are there, and so is everything the previous tile stored
     __syncthreads();
@@ -1355,7 +1365,7 @@ struct Gemm256 {
     Owed o = nothing_owed();
     o.where = (mm << 16) | mn;
     if (s.mode == kSignalNone) return o;
-    const int per_m = kMacro / g.block_m, per_n = kMacro / g.block_n;  // 1 or 2 each
+    const int per_m = g.block_m == kMacro ? 1 : 2, per_n = g.block_n == kMacro ? 1 : 2;  // plan tiles are 128 or 256 on a side here
     const int tm0 = mm * per_m, tn0 = mn * per_n;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
