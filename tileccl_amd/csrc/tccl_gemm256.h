@@ -1585,12 +1585,26 @@ struct Gemm256 {
     PullState pull = pull_begin(pa(), wg, num_wgs);
     pull_prime(pull, pa(), bgw);
     Owed unpublished = nothing_owed();
-    for (int slot = wg; slot < total; slot += num_wgs) {
-      const TileCoord c = tile_of_slot(slot, total, m);
-      if (s.mode == kSignalNone && push_offset < 0)
-        macro_tile<0>(s, c.m, c.n, pull, unpublished, src, slot == wg);
-      else
-        macro_tile<kCoherent>(s, c.m, c.n, pull, unpublished, src, slot == wg);
+    // A launch with at most one tile per workgroup does not enter the tile loop: what the compiler computes
+    // once for all tiles of a loop it computes ahead of the loop, i.e. between a workgroup's first operand
+    // requests and its first barrier, where a fused kernel already has more to do than the requests take to
+    // land (4096 x 4096 x 1024: 0.35 us per launch).  With several tiles per workgroup the loop form is the
+    // faster one (the same values would be computed between the first tile and the second).
+    if ((push_offset >= 0 || pull_offset >= 0 || reduce_offset >= 0) && total <= num_wgs) {  // (the plain GEMM has next to nothing to hoist)
+      if (wg < total) {
+        if (s.mode == kSignalNone && push_offset < 0)
+          macro_tile<0>(s, c0.m, c0.n, pull, unpublished, src, true);
+        else
+          macro_tile<kCoherent>(s, c0.m, c0.n, pull, unpublished, src, true);
+      }
+    } else {
+      for (int slot = wg; slot < total; slot += num_wgs) {
+        const TileCoord c = tile_of_slot(slot, total, m);
+        if (s.mode == kSignalNone && push_offset < 0)
+          macro_tile<0>(s, c.m, c.n, pull, unpublished, src, slot == wg);
+        else
+          macro_tile<kCoherent>(s, c.m, c.n, pull, unpublished, src, slot == wg);
+      }
     }
     if (unpublished.where >= 0) {  // the last tile: nothing follows that would wait for its stores
       wait_vmem();
