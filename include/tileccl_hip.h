@@ -201,6 +201,14 @@ int tccl_heap_destroy(void* arena);
 /* ---- small device utilities ---------------------------------------------------------- */
 /* Fill kernel (never hipMemsetAsync): signal reset, signal.py:32-40. */
 int tccl_fill_i32(int32_t* words, int64_t n, int32_t value, void* stream);
+/* Strided 2-D matrix (strides in elements, >= 0) -> dense rows of pitch ld_dst, zero-filled from
+ * (rows, cols) up to (dst_rows, dst_cols).  The reference's GEMM addresses its operands with any
+ * stride_am / stride_ak / stride_bk / stride_bn (kernels/gemm.py:63-66,139-151); the MFMA kernels here
+ * read 16-byte row vectors, so a host binding packs an operand of any other layout (a transposed
+ * A, a column slice, a K that is no multiple of the vector) with this launch first.  elem_bytes 1, 2, 4. */
+int tccl_pack_matrix(const void* src, int64_t stride_row, int64_t stride_col, int32_t rows, int32_t cols,
+                     void* dst, int64_t ld_dst, int32_t dst_rows, int32_t dst_cols, int32_t elem_bytes,
+                     void* stream);
 /* Single-word primitives, one launch each, for tests of the device semantics
  * (sync/primitives.py:357-500, tileccl_v2/ipc.py:137-254).  result: device int32[1]. */
 int tccl_prim_signal(int32_t* locks, int32_t index, void* stream);

@@ -223,7 +223,8 @@ def test_staged_allreduce_execution_policy():
 
 
 def test_b_operand_layouts():
-    """Row-major B, or the transposed view of a row-major tensor (k-major); anything else is refused."""
+    """Row-major B, or the transposed view of a row-major tensor (k-major), with rows on 16-byte boundaries, is
+    read in place; every other layout is one the launch helper packs first (None)."""
     import pytest
     import torch
 
@@ -235,12 +236,17 @@ def test_b_operand_layouts():
     W = torch.zeros(128, 64, dtype=torch.float16)  # (N, K)
     assert _launch._b_layout(W.t()) == (64, _lib.GEMM_B_KMAJOR)
     assert _launch._b_layout(torch.zeros(128, 72, dtype=torch.float16)[:, :64].t()) == (72, _lib.GEMM_B_KMAJOR)
-    assert _launch._b_layout(torch.zeros(64, 1, dtype=torch.float16)) == (1, 0)  # one column: row-major
     assert _launch._b_layout(torch.zeros(8, 1, dtype=torch.float16).t()) == (8, 0)  # (1, 8): one row, contiguous
-    with pytest.raises(ValueError, match="contiguous rows or be the transposed view"):
-        _launch._b_layout(torch.zeros(64, 256, dtype=torch.float16)[:, ::2])
+    assert _launch._b_layout(torch.zeros(64, 256, dtype=torch.float16)[:, ::2]) is None  # strided columns
+    assert _launch._b_layout(torch.zeros(64, 132, dtype=torch.float16)[:, 4:]) is None  # rows off the 16-byte grid
+    assert _launch._b_layout(torch.zeros(64, 132, dtype=torch.float16)[:, :128]) is None  # pitch no whole vector
+    assert _launch._b_layout(torch.zeros(128, 128, dtype=torch.float16)[::2, ::2].t()) is None  # strided both ways
     with pytest.raises(ValueError, match="2-D"):
-        _launch._b_layout(torch.zeros(4, 4, 4))
+        _launch.gemm_operands(torch.zeros(4, 4, dtype=torch.float16), torch.zeros(4, 4, 4, dtype=torch.float16))
+    # operands the kernels read in place pass through untouched, on any device
+    A = torch.zeros(32, 64, dtype=torch.float16)
+    a, b, k, lda, ldb, flags = _launch.gemm_operands(A, W.t())
+    assert a is A and b.data_ptr() == W.data_ptr() and (k, lda, ldb, flags) == (64, 64, 64, _lib.GEMM_B_KMAJOR)
 
 
 def test_context_and_pattern_helper_methods():

@@ -39,6 +39,31 @@ def test_gemm_allscatter_single_gpu_smoke(lib):
             heap.cleanup()
 
 
+def test_operand_views_the_reference_kernels_accept(lib):
+    """`tileccl.ops.gemm_allscatter` with a transposed A and a strided B (the reference's GEMM takes any strides,
+    /root/reference/tileccl/kernels/gemm.py:63-66): the bits of the call on contiguous copies."""
+    import tileccl_amd as tileccl
+    from tileccl_amd.memory.symmetric_heap import SymmetricHeap
+
+    heaps = SymmetricHeap.create_all(size=64 * 1024 * 1024, world_size=1)
+    try:
+        ctx = tileccl.init(backend="hip", rank=0, world_size=1, heap=heaps[0], force_backend=True)
+        a_t = seeded((72, 200), 3).cuda()  # (K, M): A is its transposed view
+        wide_b = torch.zeros(72, 2 * 136, device=ctx.device, dtype=torch.float16)
+        wide_b[:, ::2] = seeded((72, 136), 4, scale=72**-0.5).cuda()
+        for pattern in PATTERNS:
+            got = torch.zeros(200, 136, device=ctx.device, dtype=torch.float16)
+            want = torch.zeros_like(got)
+            tileccl.ops.gemm_allscatter(a_t.t(), wide_b[:, ::2], got, ctx=ctx, pattern=pattern)
+            tileccl.ops.gemm_allscatter(a_t.t().contiguous(), wide_b[:, ::2].contiguous(), want, ctx=ctx, pattern=pattern)
+            torch.cuda.synchronize()
+            assert torch.equal(bits(got), bits(want)), pattern
+            assert_gemm_close(got, a_t.t().float().cpu() @ wide_b[:, ::2].float().cpu())
+    finally:
+        for heap in heaps:
+            heap.cleanup()
+
+
 def _two_rank_case(pattern, M, K, N, dtype=torch.float16, world=2, inspect=None, **pattern_kw):
     import tileccl_amd as tileccl
     from tileccl_amd import ops

@@ -70,9 +70,18 @@ def test_fp8_needs_the_large_tile_kernel(lib):
     with pytest.raises(ValueError, match="fp8 inputs need the 256x256 kernel"):
         d = _launch.gemm_desc(A, B, out, macro_tile=128)
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
-    with pytest.raises(ValueError, match="K=72 must be a multiple of 16"):
-        d = _launch.gemm_desc(torch.zeros(256, 72, dtype=F8, device="cuda"), torch.zeros(72, 256, dtype=F8, device="cuda"), out)
+    with pytest.raises(ValueError, match="K=72 must be a multiple of 16"):  # the C ABI takes whole 16-byte vectors
+        d = _launch.gemm_desc(A, B, out)
+        d.K = 72
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    # the launch helper packs such operands (K zero-filled to 80): same bits as the padded operands passed directly
+    A72, sa = quantise((256, 72), 40)
+    B72, sb = quantise((72, 256), 41, 72**-0.5)
+    A80, B80 = torch.zeros(256, 80, dtype=F8), torch.zeros(80, 256, dtype=F8)
+    A80.view(torch.uint8)[:, :72], B80.view(torch.uint8)[:72] = A72.view(torch.uint8), B72.view(torch.uint8)
+    got72, got80 = run_gemm(lib, A72, B72, torch.bfloat16, alpha=sa * sb), run_gemm(lib, A80, B80, torch.bfloat16, alpha=sa * sb)
+    assert torch.equal(got72.view(torch.int16), got80.view(torch.int16))
+    assert_gemm_close(got72, (A72.float() @ B72.float()) * (sa * sb), rtol=5e-2, atol=1e-1, tight=0.032)
 
 
 @pytest.mark.parametrize("variant", ["s0", "s1", "s2"])

@@ -133,21 +133,28 @@ def test_unsupported_layouts_fail_loudly(lib):
 
     A, B = seeded((128, 64), 0).cuda(), seeded((64, 128), 1).cuda()
     out = torch.empty(128, 128, dtype=torch.float16, device="cuda")
-    with pytest.raises(ValueError, match="contiguous rows"):
-        _launch.gemm_desc(A, torch.empty(64, 256, dtype=torch.float16, device="cuda")[:, ::2], out)
-    with pytest.raises(ValueError, match="contiguous rows"):
-        _launch.gemm_desc(A.t().contiguous().t(), B, out)
+    with pytest.raises(ValueError, match="contiguous rows"):  # the output is written in place, never packed
+        _launch.gemm_desc(A, B, torch.empty(128, 256, dtype=torch.float16, device="cuda")[:, ::2])
     with pytest.raises(ValueError, match="leading dimension smaller"):
         d = _launch.gemm_desc(A, B, out)
         d.flags |= _lib.GEMM_B_KMAJOR  # row-major pitch (128) read as a k-major one is fine; K = 64 <= 128
         d.ldb = 32
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
-    with pytest.raises(ValueError, match="K=60 must be a multiple of 8"):
-        d = _launch.gemm_desc(A[:, :60].contiguous(), B[:60].contiguous(), out)
+    with pytest.raises(ValueError, match="K=60 must be a multiple of 8"):  # the C ABI itself takes whole vectors only
+        d = _launch.gemm_desc(A, B, out)
+        d.K = 60
+        _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="16-byte boundaries"):
+        d = _launch.gemm_desc(A, B, out)
+        d.A += 2
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
     with pytest.raises(ValueError, match="N=100 must be a multiple of 8"):
         d = _launch.gemm_desc(A, B[:, :100].contiguous(), out[:, :100].contiguous())
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
+    with pytest.raises(ValueError, match="does not fit"):
+        _lib.check(lib.tccl_pack_matrix(A.data_ptr(), 64, 1, 128, 64, out.data_ptr(), 32, 128, 64, 2, None), "tccl_pack_matrix")
+    with pytest.raises(ValueError, match="elem_bytes=3"):
+        _lib.check(lib.tccl_pack_matrix(A.data_ptr(), 64, 1, 128, 64, out.data_ptr(), 64, 128, 64, 3, None), "tccl_pack_matrix")
     with pytest.raises(ValueError, match="must be a multiple of 128x128"):
         d = _launch.gemm_desc(A, B, out, block_m=64)
         _lib.check(lib.tccl_gemm(C.byref(d), None), "tccl_gemm")
@@ -174,3 +181,87 @@ def test_every_length_of_the_k_loop(lib, macro):
         Bi = torch.randint(-2, 3, (K, 72), generator=g).half()
         want = (Ai.float() @ Bi.float()).half()
         assert torch.equal(run_gemm(lib, Ai, Bi, torch.float16, macro_tile=macro).cpu(), want), K
+
+
+@pytest.mark.parametrize("macro", MACRO)
+def test_operands_with_any_strides(lib, macro):
+    """The reference's GEMM addresses A and B with whatever strides the tensors have
+    (/root/reference/tileccl/kernels/gemm.py:63-66,139-151).  Layouts the MFMA kernels cannot read in place are
+    packed by `tccl_pack_matrix` first: the result must be the bits of the same GEMM on contiguous copies, and a
+    K that is no whole vector (zero-filled up to one) must meet the fp32 matmul like any other."""
+    from tileccl_amd import _launch, _lib
+
+    def gemm(A, B, shape):
+        out = torch.full(shape, float("nan"), dtype=torch.float16, device="cuda")
+        desc = _launch.gemm_desc(A, B, out, macro_tile=macro)
+        _lib.check(lib.tccl_gemm(C.byref(desc), _launch.stream_ptr()), "tccl_gemm")
+        torch.cuda.synchronize()
+        return out.cpu()
+
+    M, N, K = 200, 136, 104
+    A_cpu, B_cpu = seeded((M, K), 20), seeded((K, N), 21, scale=K**-0.5)
+    want = gemm(A_cpu.cuda(), B_cpu.cuda(), (M, N))
+    assert_gemm_close(want.cuda(), A_cpu.float() @ B_cpu.float(), tight=0.004)
+
+    wide_a = torch.zeros(M, 2 * K + 3, dtype=torch.float16, device="cuda")
+    wide_a[:, 3::2] = A_cpu.cuda()
+    wide_b = torch.zeros(3 * K, N + 5, dtype=torch.float16, device="cuda")
+    wide_b[::3, 5:] = B_cpu.cuda()
+    both_b = torch.zeros(2 * N, 2 * K, dtype=torch.float16, device="cuda")
+    both_b[::2, ::2] = B_cpu.t().cuda()
+    shifted_a = torch.cat([torch.zeros(1, dtype=torch.float16), A_cpu.reshape(-1)]).cuda()
+    layouts = {
+        "A transposed view": (A_cpu.t().contiguous().cuda().t(), B_cpu.cuda()),
+        "A every other column, odd offset": (wide_a[:, 3::2], B_cpu.cuda()),
+        "A rows off the 16-byte grid": (shifted_a[1:].view(M, K), B_cpu.cuda()),
+        "B every third row, columns off the grid": (A_cpu.cuda(), wide_b[::3, 5:]),
+        "B strided both ways": (A_cpu.cuda(), both_b[::2, ::2].t()),
+        "both": (A_cpu.t().contiguous().cuda().t(), both_b[::2, ::2].t()),
+    }
+    for name, (A, B) in layouts.items():
+        assert torch.equal(A.cpu(), A_cpu) and torch.equal(B.cpu(), B_cpu), name
+        got = gemm(A, B, (M, N))
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), name
+
+    # a broadcast operand (stride 0) and a K that is no multiple of 8
+    row = seeded((1, K), 22).cuda()
+    got = gemm(row.expand(M, K), B_cpu.cuda(), (M, N))
+    assert torch.equal(got.view(torch.int16), gemm(row.expand(M, K).contiguous(), B_cpu.cuda(), (M, N)).view(torch.int16))
+    for k_odd in (1, 7, 60, 101):
+        A_odd, B_odd = seeded((M, k_odd), 23 + k_odd), seeded((k_odd, N), 24 + k_odd, scale=k_odd**-0.5)
+        got = gemm(A_odd.cuda(), B_odd.cuda(), (M, N))
+        assert_gemm_close(got.cuda(), A_odd.float() @ B_odd.float(), tight=0.004)
+        k8 = (k_odd + 7) // 8 * 8
+        A_pad, B_pad = torch.zeros(M, k8, dtype=torch.float16), torch.zeros(k8, N, dtype=torch.float16)
+        A_pad[:, :k_odd], B_pad[:k_odd] = A_odd, B_odd
+        assert torch.equal(got.view(torch.int16), gemm(A_pad.cuda(), B_pad.cuda(), (M, N)).view(torch.int16))
+        got_t = gemm(A_odd.cuda(), k_major(B_odd), (M, N))  # k-major B with an odd K is packed as well
+        assert torch.equal(got_t.view(torch.int16), got.view(torch.int16))
+
+
+def test_pack_matrix_moves_every_element_once(lib):
+    """`tccl_pack_matrix` against index arithmetic on the host: 1-, 2- and 4-byte elements, both stride orders,
+    ragged patch edges, zero fill beyond the source, and a destination pitch wider than its rows."""
+    from tileccl_amd import _launch, _lib
+
+    g = torch.Generator().manual_seed(5)
+    for dtype, rows, cols, sr, sc, drows, dcols, ld in [
+        (torch.uint8, 70, 129, 300, 2, 70, 144, 144),
+        (torch.uint8, 65, 64, 1, 65, 128, 64, 80),
+        (torch.int16, 200, 104, 1, 200, 200, 104, 104),
+        (torch.int16, 1, 1, 1, 1, 3, 9, 16),
+        (torch.int32, 130, 67, 67, 1, 131, 72, 72),
+        (torch.int32, 64, 64, 0, 1, 64, 64, 64),
+    ]:
+        span = (rows - 1) * sr + (cols - 1) * sc + 1
+        backing = torch.randint(1, 100, (span,), generator=g).to(dtype).cuda()
+        src = torch.as_strided(backing, (rows, cols), (sr, sc))
+        dst = torch.full((drows, ld), 77, dtype=dtype, device="cuda")
+        rc = lib.tccl_pack_matrix(src.data_ptr(), sr, sc, rows, cols, dst.data_ptr(), ld, drows, dcols,
+                                  src.element_size(), _launch.stream_ptr())
+        _lib.check(rc, "tccl_pack_matrix")
+        torch.cuda.synchronize()
+        want = torch.full((drows, ld), 77, dtype=dtype)
+        want[:, :dcols] = 0
+        want[:rows, :cols] = src.cpu()
+        assert torch.equal(dst.cpu(), want), (dtype, rows, cols, sr, sc)

@@ -8,6 +8,7 @@ stream, like the reference's Triton launches do.
 from __future__ import annotations
 
 import ctypes as C
+import sys
 from dataclasses import dataclass, field
 
 import torch
@@ -61,22 +62,80 @@ def _row_major(t: torch.Tensor, name: str) -> int:
     return int(t.stride(0)) if t.shape[0] > 1 else int(t.shape[1])
 
 
-def _b_layout(B: torch.Tensor) -> tuple[int, int]:
-    """(ldb, flag bits) of the B operand: rows contiguous, or the ``.t()`` view of a tensor whose
-    rows are contiguous (k-major: the layout of a linear layer's weight).  The reference's kernels
-    take any strides (``/root/reference/tileccl/kernels/gemm.py:139-151``); these are the two forms
-    with 16-byte vector access."""
-    if B.ndim != 2:
-        raise ValueError(f"B must be 2-D, got {B.ndim}-D")
+def _vector_elems(t: torch.Tensor) -> int:
+    return 16 // t.element_size()
+
+
+def _rows_vectorised(t: torch.Tensor, ld: int) -> bool:
+    """Rows of pitch ``ld`` start on 16-byte boundaries (what the kernels' row vectors need)."""
+    return t.data_ptr() % 16 == 0 and ld % _vector_elems(t) == 0
+
+
+def _b_layout(B: torch.Tensor) -> tuple[int, int] | None:
+    """(ldb, flag bits) of a B operand the kernels read in place: rows contiguous, or the ``.t()``
+    view of a tensor whose rows are contiguous (k-major: the layout of a linear layer's weight).
+    ``None`` for every other layout; the reference's kernels take any strides
+    (``/root/reference/tileccl/kernels/gemm.py:139-151``) and these are the two forms with 16-byte
+    vector access."""
     K, N = B.shape
     if N == 1 or B.stride(1) == 1:
-        return _row_major(B, "B"), 0
+        ld = int(B.stride(0)) if K > 1 else int(N)
+        return (ld, 0) if ld >= N and _rows_vectorised(B, ld) else None
     if K == 1 or B.stride(0) == 1:
-        return (int(B.stride(1)) if N > 1 else int(K)), _lib.GEMM_B_KMAJOR
-    raise ValueError(
-        f"B must have contiguous rows or be the transposed view of such a tensor, got strides {tuple(B.stride())}; "
-        "call .contiguous() first"
+        ld = int(B.stride(1)) if N > 1 else int(K)
+        return (ld, _lib.GEMM_B_KMAJOR) if ld >= K and _rows_vectorised(B, ld) else None
+    return None
+
+
+_PACKED: dict[tuple, torch.Tensor] = {}
+_PACKED_LIMIT = 8
+
+
+def pack_operand(t: torch.Tensor, rows: int, cols: int, role: str) -> torch.Tensor:
+    """``t`` as a dense ``rows x cols`` matrix (zero beyond ``t``'s own shape), written by one
+    ``tccl_pack_matrix`` launch on the current stream.  The buffer is kept per (role, shape, dtype,
+    stream) and reused by the next call with that key, which the stream orders behind this one's GEMM,
+    unless a descriptor that has not been dropped yet still points at it."""
+    key = (role, rows, cols, t.dtype, t.device, stream_ptr())
+    out = _PACKED.pop(key, None)
+    if out is not None and sys.getrefcount(out) > 2:  # this name and the call's argument
+        out = None
+    if out is None:
+        while len(_PACKED) >= _PACKED_LIMIT:
+            _PACKED.pop(next(iter(_PACKED)))
+        out = torch.empty((rows, cols), dtype=t.dtype, device=t.device)
+    _PACKED[key] = out  # most recently used last
+    rc = _lib.load().tccl_pack_matrix(
+        ptr(t), int(t.stride(0)), int(t.stride(1)), int(t.shape[0]), int(t.shape[1]),
+        ptr(out), cols, rows, cols, t.element_size(), stream_ptr(),
     )
+    _lib.check(rc, f"tccl_pack_matrix[{role}]")
+    return out
+
+
+def gemm_operands(A: torch.Tensor, B: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, int, int, int, int]:
+    """(A, B, K, lda, ldb, flag bits) as the kernels read them.  An operand they can address in place
+    (16-byte row vectors: A with contiguous rows, B with contiguous rows or columns, K a whole number
+    of vectors) is passed through; any other layout the reference's pointer arithmetic accepts
+    (``/root/reference/tileccl/kernels/gemm.py:63-66,139-151``: a transposed A, strided slices, odd K)
+    is packed into a dense buffer first, K zero-filled up to the next whole vector, which adds exact zeros
+    to every dot product."""
+    for name, t in (("A", A), ("B", B)):
+        if t.ndim != 2:
+            raise ValueError(f"{name} must be 2-D, got {t.ndim}-D")
+        if any(s < 0 for s in t.stride()):
+            raise ValueError(f"{name} has negative strides {tuple(t.stride())}")
+    M, K = A.shape
+    vec = _vector_elems(A)
+    k_pad = (K + vec - 1) // vec * vec
+    lda = int(A.stride(0)) if M > 1 else int(K)
+    if k_pad != K or (K > 1 and A.stride(1) != 1) or lda < K or not _rows_vectorised(A, lda):
+        A, lda = pack_operand(A, M, k_pad, "A"), k_pad
+    layout = _b_layout(B) if k_pad == K else None
+    if layout is None:
+        N = B.shape[1]
+        B, layout = pack_operand(B, k_pad, N, "B"), (N, 0)
+    return A, B, k_pad, lda, layout[0], layout[1]
 
 
 def gemm_desc(
@@ -107,11 +166,12 @@ def gemm_desc(
         M, N = M * column_shards, N // column_shards
     if tuple(C_out.shape) != (M, N):
         raise ValueError(f"C shape mismatch: expected ({M}, {N}), got {tuple(C_out.shape)}")
+    A, B, K, lda, ldb, b_flags = gemm_operands(A, B)
     d = _lib.GemmDesc()
+    d.operands = (A, B)  # a packed operand lives as long as the descriptor
     d.A, d.B, d.C = ptr(A), ptr(B), ptr(C_out)
     d.M, d.N, d.K = int(M), int(N), int(K)
-    ldb, b_flags = _b_layout(B)
-    d.lda, d.ldb, d.ldc = _row_major(A, "A"), ldb, _row_major(C_out, "C")
+    d.lda, d.ldb, d.ldc = lda, ldb, _row_major(C_out, "C")
     d.in_dtype, d.out_dtype = dtype_code(A.dtype), dtype_code(C_out.dtype)
     d.alpha = float(alpha)
     d.block_m, d.block_n, d.group_m = int(block_m), int(block_n), int(group_m)

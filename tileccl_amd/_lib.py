@@ -135,6 +135,7 @@ SIGNATURES = {
     "tccl_heap_create": (C.c_int, [C.c_size_t, C.c_int, _P(_vp), _P(_i64)]),
     "tccl_heap_destroy": (C.c_int, [_vp]),
     "tccl_fill_i32": (C.c_int, [_vp, _i64, _i32, _vp]),
+    "tccl_pack_matrix": (C.c_int, [_vp, _i64, _i64, _i32, _i32, _vp, _i64, _i32, _i32, _i32, _vp]),
     "tccl_prim_signal": (C.c_int, [_vp, _i32, _vp]),
     "tccl_prim_signal_add": (C.c_int, [_vp, _i32, _i32, _vp, _vp]),
     "tccl_prim_try_wait": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp]),

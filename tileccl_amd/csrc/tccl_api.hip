@@ -151,6 +151,27 @@ __global__ void fill_kernel(int32_t* w, int64_t n, int32_t v) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) w[i] = v;
 }
 
+// Strided matrix -> dense rows, one 64 x 64 patch per workgroup through LDS: the patch is read along
+// whichever source index is closer in memory and written along the destination's rows, so both sides
+// move whole lines whatever the source's strides are.  Elements outside the source are written as zero.
+template <typename T>
+__global__ __launch_bounds__(256) void pack_kernel(const T* src, int64_t stride_row, int64_t stride_col, int rows, int cols,
+                                                   T* dst, int64_t ld_dst, int dst_rows, int dst_cols) {
+  __shared__ T patch[64][65];
+  const int r0 = (int)blockIdx.y * 64, c0 = (int)blockIdx.x * 64;
+  const int fast = (int)threadIdx.x & 63, slow = (int)threadIdx.x >> 6;
+  const bool along_cols = stride_col <= stride_row;
+  for (int i = slow; i < 64; i += 4) {
+    const int r = along_cols ? i : fast, c = along_cols ? fast : i;
+    T v = 0;
+    if (r0 + r < rows && c0 + c < cols) v = src[(int64_t)(r0 + r) * stride_row + (int64_t)(c0 + c) * stride_col];
+    patch[r][c] = v;
+  }
+  __syncthreads();
+  for (int i = slow; i < 64; i += 4)
+    if (r0 + i < dst_rows && c0 + fast < dst_cols) dst[(int64_t)(r0 + i) * ld_dst + c0 + fast] = patch[i][fast];
+}
+
 __global__ void prim_signal_kernel(int32_t* locks, int i) { tccl::tile_signal(locks, i); }
 __global__ void prim_signal_add_kernel(int32_t* w, int i, int v, int32_t* res) { *res = tccl::tile_signal_add(w, i, v); }
 __global__ void prim_try_wait_kernel(int32_t* locks, int i, int spins, int consume, int32_t* res) {
@@ -876,6 +897,31 @@ int tccl_fill_i32(int32_t* words, int64_t n, int32_t value, void* stream) {
   int blocks = (int)((n + 255) / 256);
   if (blocks > 1024) blocks = 1024;
   hipLaunchKernelGGL(fill_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, words, n, value);
+  TCCL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tccl_pack_matrix(const void* src, int64_t stride_row, int64_t stride_col, int32_t rows, int32_t cols, void* dst,
+                     int64_t ld_dst, int32_t dst_rows, int32_t dst_cols, int32_t elem_bytes, void* stream) {
+  if (dst_rows <= 0 || dst_cols <= 0) return 0;
+  if (!src || !dst) return fail(TCCL_ERR_INVALID, "pack_matrix: NULL pointer");
+  if (rows < 0 || cols < 0 || rows > dst_rows || cols > dst_cols || stride_row < 0 || stride_col < 0 || ld_dst < dst_cols)
+    return fail(TCCL_ERR_INVALID, "pack_matrix: source %dx%d (strides %lld, %lld) does not fit a %dx%d destination of pitch %lld",
+                rows, cols, (long long)stride_row, (long long)stride_col, dst_rows, dst_cols, (long long)ld_dst);
+  const dim3 grid((unsigned)((dst_cols + 63) / 64), (unsigned)((dst_rows + 63) / 64));
+  if (grid.y > 65535u) return fail(TCCL_ERR_UNSUPPORTED, "pack_matrix: more than 65535 x 64 rows");
+  const hipStream_t st = (hipStream_t)stream;
+  if (elem_bytes == 1)
+    hipLaunchKernelGGL(pack_kernel<uint8_t>, grid, dim3(256), 0, st, (const uint8_t*)src, stride_row, stride_col, rows, cols,
+                       (uint8_t*)dst, ld_dst, dst_rows, dst_cols);
+  else if (elem_bytes == 2)
+    hipLaunchKernelGGL(pack_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t*)src, stride_row, stride_col, rows, cols,
+                       (uint16_t*)dst, ld_dst, dst_rows, dst_cols);
+  else if (elem_bytes == 4)
+    hipLaunchKernelGGL(pack_kernel<uint32_t>, grid, dim3(256), 0, st, (const uint32_t*)src, stride_row, stride_col, rows, cols,
+                       (uint32_t*)dst, ld_dst, dst_rows, dst_cols);
+  else
+    return fail(TCCL_ERR_INVALID, "pack_matrix: elem_bytes=%d must be 1, 2 or 4", elem_bytes);
   TCCL_HIP(hipGetLastError());
   return 0;
 }
