@@ -592,6 +592,57 @@ def probe_mfma_table(repeats=3):
     return {"probe": "tccl_mfma_rate_probe", "workgroups": runs[0]["workgroups"], "table": table}
 
 
+def probe_copy_table(steps=50):
+    """What a copy (every byte read once and written once) reaches on this part, by four different kernels: the
+    library's `tccl_copy_block` (the loops S0's exchange phase runs), torch's tensor copy (the runtime's
+    device-to-device copy), a torch elementwise kernel (`add(src, 0)`), and `tccl_exchange_rows` at c1's shape
+    (S0's exchange phase itself, both emulated ranks' blocks).  GB/s counts bytes read plus bytes written."""
+    import ctypes as C
+
+    import torch
+
+    from tileccl_amd import _launch, _lib
+    from tileccl_amd.memory.symmetric_heap import SymmetricHeap
+    from tileccl_amd.primitives import communication
+
+    lib = _lib.load()
+    table = {}
+    heaps = SymmetricHeap.create_all(size=1536 << 20, world_size=2)
+    try:
+        h = heaps[0]
+        for mib in (32, 64, 512):
+            n = mib << 20
+            src, dst = h.allocate_tensor((n // 2,), torch.float16), h.allocate_tensor((n // 2,), torch.float16)
+            src.normal_()
+            runs = {
+                "tccl_copy_block": lambda _v, src=src, dst=dst: communication.copy_block(dst, src, h, src_rank=0, dst_ranks=(0,)),
+                "torch copy_": lambda _v, src=src, dst=dst: dst.copy_(src),
+                "torch add(src, 0)": lambda _v, src=src, dst=dst: torch.add(src, 0, out=dst),
+            }
+            for name, run in runs.items():
+                _, ms = time_variant(run, "copy", steps, 5)
+                assert torch.equal(dst, src), name
+                table[f"{name} {mib} MiB"] = {"us": round(ms * 1e3, 2), "gbs": round(2 * n / (ms * 1e-3) / 1e9, 1)}
+        M, N = WORKLOADS["c1"][1], WORKLOADS["c1"][2]
+        outs = [hp.allocate_tensor((2 * M, N), torch.float16) for hp in heaps]
+        for r, o in enumerate(outs):
+            o[r * M:(r + 1) * M].normal_()
+        views = [_launch.heap_view(hp.get_heap_bases(), r, 2) for r, hp in enumerate(heaps)]
+        transport = _launch.transport_desc(_lib.DIR_PUSH | _lib.DIR_PULL, 16384, None, 0)
+
+        def exchange(_v):
+            rc = lib.tccl_exchange_rows(_launch.ptr(outs[0]), M, N, N, 2, C.byref(views[0]), C.byref(transport), _launch.stream_ptr())
+            _lib.check(rc, "tccl_exchange_rows")
+
+        _, ms = time_variant(exchange, "copy", steps, 5)
+        moved = 2 * M * N * 2  # this rank's block pushed, the peer's block pulled
+        table["tccl_exchange_rows c1 (2 x 32 MiB moved)"] = {"us": round(ms * 1e3, 2), "gbs": round(2 * moved / (ms * 1e-3) / 1e9, 1)}
+    finally:
+        for hp in heaps:
+            hp.cleanup()
+    return {"probe": "copy", "peak_gbs": PEAK_HBM_GBS, "table": table}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -613,6 +664,9 @@ def main() -> int:
                          "as its .t() view (a linear layer's weight)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-live-pair", action="store_true", help="skip the two-live-ranks leg (all-gather workloads)")
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="only time stand-alone copies (the library's copy loops, torch's copy and an elementwise "
+                         "kernel, S0's exchange phase at c1's shape) and print the table as one JSON line")
     ap.add_argument("--probe-mfma", action="store_true",
                     help="only run the MFMA-rate probe (every instruction shape, on zeros and on normally distributed "
                          "operands) and print its table as one JSON line")
@@ -628,6 +682,9 @@ def main() -> int:
     _lib.load()
     if args.probe_mfma:
         print(json.dumps(probe_mfma_table()))
+        return 0
+    if args.probe_copy:
+        print(json.dumps(probe_copy_table()))
         return 0
     props = get_backend().get_device_properties()
     if WORKLOADS[args.workload][0] == "ch":

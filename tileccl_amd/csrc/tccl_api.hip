@@ -131,6 +131,18 @@ __global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
   tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
 }
 
+// The stand-alone bulk kernels (S0's second kernel, the scatter / gather / block copies, the stand-alone
+// reduction): the communication role with everything else compiled out.  The full role is a large kernel,
+// and a launch of it takes 1.2 us longer to move the same bytes (c1's 128 MiB exchange: 21.5 -> 20.3 us).
+__global__ __launch_bounds__(256) void copy_kernel(tccl::CommArgs c) {
+  __shared__ int word[4];
+  tccl::comm_role<tccl::kThreadsComm, tccl::kBulkCopy>(c, (int)blockIdx.x, (int)gridDim.x, word);
+}
+__global__ __launch_bounds__(256) void reduce_kernel(tccl::CommArgs c) {
+  __shared__ int word[4];
+  tccl::comm_role<tccl::kThreadsComm, tccl::kBulkReduce>(c, (int)blockIdx.x, (int)gridDim.x, word);
+}
+
 // Staged collectives: workgroup w carries slot w % slots of the (w / slots)-th rank named in a.ranks.
 __global__ __launch_bounds__(256) void staged_kernel(tccl::StagedArgs a) {
   __shared__ int word;
@@ -568,15 +580,26 @@ int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
   const int span = check_comm_span(c);
   if (span) return span;
   if (wgs < 1) wgs = 1;
-  hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
+  if (c.granularity != tccl::kBulk)
+    hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
+  else if (c.op == tccl::kOpReduceScatter)
+    hipLaunchKernelGGL(reduce_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
+  else
+    hipLaunchKernelGGL(copy_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
   TCCL_HIP(hipGetLastError());
   return 0;
 }
 
-// Workgroups of a stand-alone bulk kernel.  Swept at 2 / 4 / 8 / 16 per CU on the 128 MiB
-// exchange of the 4096 x 4096 x 1024 all-gather (27.2 / 25.5 / 26.0 / 27.7 us) and on the
-// reductions of the reduce-scatter configurations (4 per CU ahead of 8 by 3-4 %).
-int bulk_comm_wgs(const tccl_device_info& dev) { return dev.compute_units * 4; }
+// Workgroups of a stand-alone bulk kernel, per CU: 8 for copies, 4 for reductions.  Swept on the 128 MiB
+// exchange of the 4096 x 4096 x 1024 all-gather (2 / 4 / 8 per CU: 20.7 / 20.3 / 19.7 us; tasks of 128 KiB
+// instead of 32 KiB: 21.7 us) and on the reductions of the reduce-scatter configurations (4 per CU ahead
+// of 8 by 3-4 %).
+#ifndef TCCL_BULK_COPY_WGS
+#define TCCL_BULK_COPY_WGS 8
+#endif
+int bulk_comm_wgs(const tccl_device_info& dev, const tccl::CommArgs& c) {
+  return dev.compute_units * (c.op == tccl::kOpReduceScatter ? 4 : TCCL_BULK_COPY_WGS);
+}
 
 // The second kernel of S0 waits for nothing, so a plan's TileGroups mean nothing to it: it
 // sweeps the whole block (a reduce-scatter: each owner's shard) as one run of tasks.  Cut
@@ -654,7 +677,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
       if (rc) return rc;
       make_bulk(&c);
       if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
-      return launch_comm(c, bulk_comm_wgs(dev), stream);
+      return launch_comm(c, bulk_comm_wgs(dev, c), stream);
     }
     Fused256Args f;
     f.g = g;
@@ -698,7 +721,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
     if (rc) return rc;
     make_bulk(&c);
     if (c.world <= 1 && c.op != tccl::kOpReduceScatter) return 0;
-    return launch_comm(c, bulk_comm_wgs(dev), stream);
+    return launch_comm(c, bulk_comm_wgs(dev, c), stream);
   }
   int comm = tr && tr->num_comm_wgs > 0 ? tr->num_comm_wgs : dev.compute_units;
   s.epoch = sync->epoch > 0 ? sync->epoch : 1;
@@ -1020,7 +1043,7 @@ int tccl_scatter_cols(const void* C, int32_t M, int64_t ldc, int32_t elem_bytes,
   c.dst_ld = sc->dst_ld;
   c.dst_col_off = sc->dst_col_offset;
   if ((rc = set_task_units(&c, nullptr, false))) return rc;
-  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+  return launch_comm(c, bulk_comm_wgs(dev, c), (hipStream_t)stream);
 }
 
 int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, int32_t elem_bytes,
@@ -1054,7 +1077,7 @@ int tccl_exchange_rows(void* out, int32_t rows_per_rank, int32_t N, int64_t ld, 
   c.out = (char*)out;
   c.ld_out_bytes = ld * elem_bytes;
   if ((rc = set_task_units(&c, tr, false))) return rc;
-  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+  return launch_comm(c, bulk_comm_wgs(dev, c), (hipStream_t)stream);
 }
 
 int tccl_copy_block(void* dst, uint32_t dst_ranks, const void* src, int32_t src_rank, int32_t rows, int64_t row_bytes,
@@ -1096,7 +1119,7 @@ int tccl_copy_block(void* dst, uint32_t dst_ranks, const void* src, int32_t src_
   c.copy_dst_ranks = dst_ranks;
   // 32 KiB per task, whatever the element type of the caller's data
   c.copy_units = c.reduce_units = 2048;
-  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+  return launch_comm(c, bulk_comm_wgs(dev, c), (hipStream_t)stream);
 }
 
 int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int64_t ld_shard, int32_t M,
@@ -1135,7 +1158,7 @@ int tccl_gather_cols(void* gathered, int64_t ld_gathered, const void* shard, int
   c.out = (char*)gathered;
   c.ld_out_bytes = ld_gathered * elem_bytes;
   if ((rc = set_task_units(&c, tr, false))) return rc;
-  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+  return launch_comm(c, bulk_comm_wgs(dev, c), (hipStream_t)stream);
 }
 
 static int fill_reduce(tccl::CommArgs* c, const void* partial, int partial_dtype, void* out, int out_dtype, int64_t ld_out,
@@ -1190,7 +1213,7 @@ int tccl_reduce_rows(const void* partial, int32_t partial_dtype, int64_t ld_part
   if ((rc = fill_reduce(&c, partial, partial_dtype, out, out_dtype, ld_out, M, N, heap->world_size, emulate_peer, true))) return rc;
   c.granularity = tccl::kBulk;
   if ((rc = set_task_units(&c, tr, true))) return rc;
-  return launch_comm(c, bulk_comm_wgs(dev), (hipStream_t)stream);
+  return launch_comm(c, bulk_comm_wgs(dev, c), (hipStream_t)stream);
 }
 
 static int allscatter_impl(const tccl_gemm_desc* d, const tccl_scatter_desc* sc, const tccl_heap_view* heap,

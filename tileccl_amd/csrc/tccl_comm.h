@@ -107,7 +107,6 @@ template <int kPolicy>
 TCCL_D void st16(__amdgpu_buffer_rsrc_t w, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, w, off, 0, kPolicy); }
 
 constexpr int kThreadsComm = 256;  // threads of a stand-alone communication workgroup
-constexpr int kCommUnroll = 8;     // 16-byte accesses a thread keeps in flight
 // Cache policy of the stand-alone bulk kernels (the second kernel of S0), measured on the
 // 128 MiB exchange that follows the 4096 x 4096 x 1024 GEMM and on the reductions of the
 // reduce-scatter configurations: plain (write-back) accesses for copies, 25.5 us against
@@ -119,18 +118,20 @@ constexpr int kBulkReducePolicy = kStreaming;
 // kPolicy is the cache policy of both sides: kCoherent inside fused launches (the source
 // was just written by other workgroups, the target will be read by a peer), kStreaming
 // for the stand-alone bulk kernel.
+constexpr int kCopyHalf = 4;  // 16-byte accesses per thread in one of the two register sets
+
 template <int kPolicy, int kThreads>
-TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
-  const int tid = threadIdx.x;
-  const int src_rank = __builtin_ctz(x.src_ranks);
-  const __amdgpu_buffer_rsrc_t src = window(a.heap_bases[src_rank] + x.src_off);
-  const bool flat = (x.src_pitch == (int64_t)x.upr * 16) && (x.dst_pitch == x.src_pitch);
-  const uint32_t sp = (uint32_t)x.src_pitch, dp = (uint32_t)x.dst_pitch;
-  for (int u0 = u_lo; u0 < u_hi; u0 += kThreads * kCommUnroll) {
-    u32x4 v[kCommUnroll];
-    uint32_t doff[kCommUnroll];
+struct CopyBatch {
+  const CommArgs& a;
+  const Xfer& x;
+  __amdgpu_buffer_rsrc_t src;
+  bool flat;
+  uint32_t sp, dp;
+  int tid, u_hi;
+
+  TCCL_D void load(int u0, u32x4 (&v)[kCopyHalf], uint32_t (&doff)[kCopyHalf]) const {
 #pragma unroll
-    for (int k = 0; k < kCommUnroll; ++k) {
+    for (int k = 0; k < kCopyHalf; ++k) {
       const int u = u0 + tid + k * kThreads;
       uint32_t soff;
       if (flat) {
@@ -144,13 +145,44 @@ TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
       if (u >= u_hi) soff = 0;  // idle lane: harmless re-read of the first unit, nothing stored
       v[k] = ld16<kPolicy>(src, soff);
     }
+  }
+  TCCL_D void store(int u0, const u32x4 (&v)[kCopyHalf], const uint32_t (&doff)[kCopyHalf]) const {
     for (int q = 0; q < a.world; ++q) {
       if (!((x.dst_ranks >> q) & 1u)) continue;
       const __amdgpu_buffer_rsrc_t dst = window(a.heap_bases[q] + x.dst_off);
 #pragma unroll
-      for (int k = 0; k < kCommUnroll; ++k)
+      for (int k = 0; k < kCopyHalf; ++k)
         if (u0 + tid + k * kThreads < u_hi) st16<kPolicy>(dst, doff[k], v[k]);
     }
+  }
+};
+
+// Two register sets per thread, one being stored while the other is being loaded: from the second batch
+// on a wavefront always has loads and stores in flight together, so the memory system sees reads and writes
+// mixed instead of a read phase and a write phase (all workgroups of a launch start together and would
+// otherwise alternate in step).
+template <int kPolicy, int kThreads>
+TCCL_D void run_copy(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  const int src_rank = __builtin_ctz(x.src_ranks);
+  const CopyBatch<kPolicy, kThreads> b{a, x, window(a.heap_bases[src_rank] + x.src_off),
+                                       (x.src_pitch == (int64_t)x.upr * 16) && (x.dst_pitch == x.src_pitch),
+                                       (uint32_t)x.src_pitch, (uint32_t)x.dst_pitch, (int)threadIdx.x, u_hi};
+  constexpr int kBatch = kThreads * kCopyHalf;
+  u32x4 v0[kCopyHalf], v1[kCopyHalf];
+  uint32_t d0[kCopyHalf], d1[kCopyHalf];
+  int u0 = u_lo;
+  if (u0 >= u_hi) return;
+  b.load(u0, v0, d0);
+  for (;;) {
+    const int u1 = u0 + kBatch;
+    if (u1 < u_hi) b.load(u1, v1, d1);
+    b.store(u0, v0, d0);
+    if (u1 >= u_hi) break;
+    const int u2 = u1 + kBatch;
+    if (u2 < u_hi) b.load(u2, v0, d0);
+    b.store(u1, v1, d1);
+    if (u2 >= u_hi) break;
+    u0 = u2;
   }
 }
 
@@ -282,8 +314,19 @@ TCCL_D void run_reduce(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
   }
 }
 
-template <int kThreads>
+// kOnly names what a stand-alone bulk kernel is compiled for (kAllRoles: everything, fused launches included).
+enum BulkOnly { kAllRoles = 0, kBulkCopy = 1, kBulkReduce = 2 };
+
+template <int kThreads, int kOnly = kAllRoles>
 TCCL_D void run_xfer(const CommArgs& a, const Xfer& x, int u_lo, int u_hi) {
+  if constexpr (kOnly == kBulkCopy) {
+    run_copy<kBulkCopyPolicy, kThreads>(a, x, u_lo, u_hi);
+    return;
+  }
+  if constexpr (kOnly == kBulkReduce) {
+    if (x.reduce) run_reduce<kBulkReducePolicy, kThreads>(a, x, u_lo, u_hi);
+    return;
+  }
   const bool fused = a.granularity != kBulk;
   if (x.reduce) {
     if (fused)
@@ -468,7 +511,7 @@ TCCL_D bool rs_not_mine(const CommArgs& a, int row) {
 // sources are ready or soon will be, independent of this rank's GEMM), then pushes /
 // reductions in production order.  Workgroup w takes tasks w, w + n, w + 2n, ...; no
 // GEMM workgroup ever waits on a communication workgroup, so the order is deadlock-free.
-template <int kThreads = kThreadsComm>
+template <int kThreads = kThreadsComm, int kOnly = kAllRoles>
 TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
   if (a.op == kOpNone || num_wgs <= 0) return;
   Waiter wait{a, lds_word, now_ticks() + a.spin_ticks};
@@ -479,7 +522,7 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
   const int unit_elems = is_rs ? 8 : 16 / a.esize;
   const int units_per_task = is_rs ? a.reduce_units : a.copy_units;
 
-  if (a.granularity == kPerTile) {
+  if (kOnly == kAllRoles && a.granularity == kPerTile) {
     const int total = a.tile_rows * a.tile_cols;
     const int n_pull = do_pull ? peers * total : 0;
     const int n_all = n_pull + (do_push ? total : 0);
@@ -534,7 +577,7 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
     if (g >= a.n_groups) break;
     if (rs_not_mine(a, group_lo(a, g))) continue;
     bool ok = true;
-    if (a.granularity == kPerGroup) {
+    if (kOnly == kAllRoles && a.granularity == kPerGroup) {
       uint32_t ranks = pull ? (1u << peer) : (is_rs ? all_ranks(a.world) : (1u << a.rank));
       ok = wait.group(g, ranks);
     }
@@ -543,9 +586,9 @@ TCCL_D void comm_role(const CommArgs& a, int wg, int num_wgs, int* lds_word) {
       const int units = x.rows * x.upr;
       const int lo = local * units_per_task;
       const int hi = lo + units_per_task < units ? lo + units_per_task : units;
-      if (lo < hi) run_xfer<kThreads>(a, x, lo, hi);
+      if (lo < hi) run_xfer<kThreads, kOnly>(a, x, lo, hi);
     }
-    if (a.granularity == kPerGroup) task_done(a, g, tasks_g * tasks_factor);
+    if (kOnly == kAllRoles && a.granularity == kPerGroup) task_done(a, g, tasks_g * tasks_factor);
   }
 }
 
