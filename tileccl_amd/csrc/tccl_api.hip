@@ -126,14 +126,10 @@ __global__ __launch_bounds__(256, 2) void gemm128_kernel(tccl::GemmArgs g) {
 #endif
 }
 
-__global__ __launch_bounds__(256) void comm_kernel(tccl::CommArgs c) {
-  __shared__ int word[4];
-  tccl::comm_role(c, (int)blockIdx.x, (int)gridDim.x, word);
-}
-
 // The stand-alone bulk kernels (S0's second kernel, the scatter / gather / block copies, the stand-alone
-// reduction): the communication role with everything else compiled out.  The full role is a large kernel,
-// and a launch of it takes 1.2 us longer to move the same bytes (c1's 128 MiB exchange: 21.5 -> 20.3 us).
+// reduction): the communication role with everything else compiled out.  The full role (per-tile and
+// per-group waits, every reduction type) is a large kernel, and a launch of it took 1.2 us longer to move
+// the same bytes (the 128 MiB exchange of the 4096 x 4096 x 1024 all-gather: 21.5 against 20.3 us).
 __global__ __launch_bounds__(256) void copy_kernel(tccl::CommArgs c) {
   __shared__ int word[4];
   tccl::comm_role<tccl::kThreadsComm, tccl::kBulkCopy>(c, (int)blockIdx.x, (int)gridDim.x, word);
@@ -580,9 +576,8 @@ int launch_comm(const tccl::CommArgs& c, int wgs, hipStream_t stream) {
   const int span = check_comm_span(c);
   if (span) return span;
   if (wgs < 1) wgs = 1;
-  if (c.granularity != tccl::kBulk)
-    hipLaunchKernelGGL(comm_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
-  else if (c.op == tccl::kOpReduceScatter)
+  if (c.granularity != tccl::kBulk) return fail(TCCL_ERR_INVALID, "a stand-alone communication launch is a bulk one");
+  if (c.op == tccl::kOpReduceScatter)
     hipLaunchKernelGGL(reduce_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
   else
     hipLaunchKernelGGL(copy_kernel, dim3(wgs), dim3(tccl::kThreadsComm), 0, stream, c);
