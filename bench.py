@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # this script scaled by what the same counters read for the bulk copy kernel of known size
 # (profiles/fused256_kernel_<workload>_s2_counters.md).  Known only for the default tile choice.
 MEASURED_TRAFFIC_BYTES = {("c1", "s2", 0): int(176.2 * 2**20), ("c2", "s2", 0): int(352.0 * 2**20),
-                          ("c3", "s2", 0): int(447.9 * 2**20), ("c4", "s2", 0): int(575.6 * 2**20)}
+                          ("c3", "s2", 0): int(447.9 * 2**20), ("c4", "s2", 0): int(513.3 * 2**20)}
 
 WORKLOADS = {
     # name: kind, local M, N, K, block_m, input type

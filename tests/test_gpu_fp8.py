@@ -188,9 +188,9 @@ def test_baseline_config_4_properties(lib, own_rows):
 @pytest.mark.parametrize("variant", ["s1", "s2"])
 @pytest.mark.parametrize("world,M", [(2, 1024), (3, 768)])
 def test_fp8_own_rows_kept_in_registers_give_the_same_bytes(lib, variant, world, M):
-    """fp8 inputs with the owned rows' partial kept in the accumulators: the fp8 kernels reduce
-    the other owners' rows by reading the stored partial back (a third code path next to the
-    two of the 16-bit kernels).  Outputs equal the oracle's reduction of the partials a plain
+    """fp8 inputs with the owned rows' partial kept in the accumulators: with two ranks the other
+    owner's rows are reduced from the accumulators as well (the stored, rounded partial enters the
+    sum), with three they are reduced by reading the stored partial back.  Outputs equal the oracle's reduction of the partials a plain
     run stored, bit for bit (three ranks: order-sensitive magnitudes); the owned rows of
     `partial` are never written, the other rows are."""
     from tileccl_amd.v2 import FusedGemmReduceScatter, SymmetricHeap

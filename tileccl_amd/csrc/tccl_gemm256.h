@@ -1217,8 +1217,7 @@ struct Gemm256 {
           // idle lanes re-read the tile's first chunk and store nothing
           src[r] = live[r] ? (uint32_t)((lrow * g.ldc + lcol) * kEsz) : 0u;
           dst[r] = (uint32_t)((lrow * ld_out + lcol) * 2);
-          if constexpr (!kFp8)
-            if (store_partial && live[r]) __builtin_amdgcn_raw_buffer_store_b128(v, r_mine, src[r], 0, kCoherent);
+          if (store_partial && live[r]) __builtin_amdgcn_raw_buffer_store_b128(v, r_mine, src[r], 0, kCoherent);
           int n;
           unpack(v, sum[r], n);
         }
@@ -1333,10 +1332,12 @@ struct Gemm256 {
       if (ra->active && ra->own_in_registers) {
         const int owner = row0 / ra->shard_rows;
         // The other owner's rows, reduced on its behalf (emulation, two ranks): the partial is
-        // stored as that owner would read it, and the same registers enter its sum.
-        // (Not in the fp8 kernels: the extra code costs them more in spilled registers than the
-        // saved read-back is worth, measured +4 % at 16384x4096x2048.)
-        const bool for_peer = !kFp8 && owner != ra->rank && ra->emulate_peer && ra->world == 2;
+        // stored as that owner would read it, and the same registers enter its sum (the staged,
+        // rounded values: the bits of a sum that read the stored partial back).
+        // (The fp8 kernels once read the partial back instead: this path cost them registers they kept in
+        // scratch memory inside the K loops, +4 % at 16384x4096x2048; with the wavefront number and the LDS
+        // addresses in scalar registers they have the room, and the saved read-back is worth 6 %.)
+        const bool for_peer = owner != ra->rank && ra->emulate_peer && ra->world == 2;
         if ((owner == ra->rank || for_peer) && reduce_wait(ra, s, mm, mn)) {
           epilogue_reduce(ra, row0, col0, acc, owner, for_peer);
           unpublished = publish_lookup(s, mm, mn);
