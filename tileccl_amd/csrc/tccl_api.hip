@@ -380,15 +380,18 @@ int launch_fused(int in_dtype, int out_dtype, const tccl::GemmArgs& g, const tcc
 // ---- large-tile path ----------------------------------------------------------------------------
 
 // 256 x 256 tiles pay off once there are enough of them to occupy most CUs; below that
-// the 128 x 128 kernel spreads the work over more workgroups.
-bool use_macro(const tccl_gemm_desc* d, const tccl_device_info& dev) {
+// the 128 x 128 kernel spreads the work over more workgroups.  With large tiles on exactly half of the CUs
+// the GEMM alone is 5-6 % faster on small tiles (2048 x 4096 x 1024: 22.3 against 23.3 us; 4096 x 2048 x 2048:
+// 38.1 against 40.6; 96 large tiles: 63.3 against 73.8), from 144 large tiles on it is slower (3072^3: 76.6
+// against 58.5 us); the fused launches keep the large tiles there (their transfers ride on the K loops).
+bool use_macro(const tccl_gemm_desc* d, const tccl_device_info& dev, bool fused = true) {
   if (d->in_dtype == TCCL_F8E4M3) return true;  // fp8 exists only as the large-tile kernel (check_gemm vets the plan tile)
   if (!plan_tile_fits_macro(d)) return false;
   if (d->column_shards > 1 && (d->M / d->column_shards) % 256) return false;  // a tile must not straddle two row blocks
   if (d->macro_tile == 128) return false;
   if (d->macro_tile == 256) return true;
   const int64_t tiles = (int64_t)((d->M + 255) / 256) * ((d->N + 255) / 256);
-  return tiles * 2 >= dev.compute_units;
+  return fused ? tiles * 2 >= dev.compute_units : tiles * 2 > dev.compute_units;
 }
 
 tccl::Macro build_macro(const tccl_gemm_desc* d, const tccl_device_info& dev, int num_wgs) {
@@ -664,7 +667,7 @@ int run_variant(const tccl_gemm_desc* d, tccl::CommArgs& c, const tccl_sync_desc
   tccl::SignalArgs s;
   memset(&s, 0, sizeof s);
   int64_t* trace_start = sync ? sync->trace_start_clock : nullptr;
-  if (use_macro(d, dev)) {
+  if (use_macro(d, dev, variant != TCCL_S0_BULK)) {
     const int wgs = default_macro_wgs(d, dev);
     const tccl::Macro m = build_macro(d, dev, wgs);
     if (variant == TCCL_S0_BULK) {
@@ -982,7 +985,7 @@ int tccl_gemm(const tccl_gemm_desc* d, void* stream) {
   build_gemm_args(d, dev, &g);
   tccl::SignalArgs s;
   memset(&s, 0, sizeof s);
-  if (use_macro(d, dev)) {
+  if (use_macro(d, dev, false)) {
     const int wgs = default_macro_wgs(d, dev);
     return launch_gemm256(d->in_dtype, d->out_dtype, g, build_macro(d, dev, wgs), wgs, (hipStream_t)stream);
   }
