@@ -97,8 +97,8 @@ def test_static_words_give_the_bytes_of_caller_supplied_words(lib, variant, macr
 @pytest.mark.parametrize("variant", ["s1", "s2"])
 @pytest.mark.parametrize("macro", [128, 256])
 def test_a_puller_ahead_of_its_peer_waits_and_gives_up(lib, variant, macro):
-    """Round 1 in order (push, then pull).  In round 2 the puller is issued BEFORE the pusher: the peer's words
-    still hold round 1's values, which must not satisfy round 2; the puller's bounded wait expires, it raises its
+    """Call 1 in order (push, then pull).  In call 2 the puller is issued BEFORE the pusher: the peer's words
+    still hold the values of call 1, which must not satisfy call 2; the puller's bounded wait expires, it raises its
     fault word and leaves the peer's rows of its output alone.  Nothing hangs: the wait is the kernel's own.
     Once the pusher has caught up (and made the call the puller gave up on), the next round works again."""
     from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
@@ -113,31 +113,31 @@ def test_a_puller_ahead_of_its_peer_waits_and_gives_up(lib, variant, macro):
         A1, B1 = into_heap(heaps[1], seeded((M, K), 3)), into_heap(heaps[1], seeded((K, N), 4, scale=K**-0.5))
         for o in (puller, pusher):
             o.out.zero_()
-        launch_static(lib, pusher, A1, B1, variant)  # round 1
+        launch_static(lib, pusher, A1, B1, variant)  # call 1
         launch_static(lib, puller, A0, B0, variant)
         puller.check_faults()
         pusher.check_faults()
         first = pusher.out[M:].clone()
         assert torch.equal(bits(puller.out[M:]), bits(first)) and torch.count_nonzero(first).item() > 0
 
-        A1.copy_(seeded((M, K), 5))  # round 2: new inputs on the pushing rank ...
+        A1.copy_(seeded((M, K), 5))  # call 2: new inputs on the pushing rank ...
         puller.out[M:].fill_(-3.0)  # ... and a marker where its block would land
         launch_static(lib, puller, A0, B0, variant, spin_limit_ns=200_000)  # ahead of its peer
         torch.cuda.synchronize()
-        assert int(puller.words.fault.item()) != 0, "round 1's words satisfied round 2"
+        assert int(puller.words.fault.item()) != 0, "the words of call 1 satisfied call 2"
         with pytest.raises(RuntimeError):
             puller.check_faults()
         assert torch.all(puller.out[M:] == -3.0), "rows were pulled although the peer had not produced them"
         assert_gemm_close(puller.out[:M], A0.float().cpu() @ B0.float().cpu(), tight=0.004)  # its own block is there
         puller.words.fault.zero_()
 
-        launch_static(lib, pusher, A1, B1, variant)  # the peer's round 2 (nobody waits for it any more)
-        launch_static(lib, pusher, A1, B1, variant)  # round 3, in order again
+        launch_static(lib, pusher, A1, B1, variant)  # the peer's call 2 (nobody waits for it any more)
+        launch_static(lib, pusher, A1, B1, variant)  # call 3, in order again
         launch_static(lib, puller, A0, B0, variant)
         puller.check_faults()
         pusher.check_faults()
         assert torch.equal(bits(puller.out[M:]), bits(pusher.out[M:]))
-        assert not torch.equal(bits(pusher.out[M:]), bits(first))  # round 3 moved the new bytes
+        assert not torch.equal(bits(pusher.out[M:]), bits(first))  # call 3 moved the new bytes
     finally:
         for h in heaps:
             h.cleanup()
