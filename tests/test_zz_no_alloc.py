@@ -100,7 +100,7 @@ def test_a_puller_ahead_of_its_peer_waits_and_gives_up(lib, variant, macro):
     """Call 1 in order (push, then pull).  In call 2 the puller is issued BEFORE the pusher: the peer's words
     still hold the values of call 1, which must not satisfy call 2; the puller's bounded wait expires, it raises its
     fault word and leaves the peer's rows of its output alone.  Nothing hangs: the wait is the kernel's own.
-    Once the pusher has caught up (and made the call the puller gave up on), the next round works again."""
+    Once the pusher has caught up (and made the call the puller gave up on), the next call works again."""
     from tileccl_amd.v2 import FusedGemmAllGather, SymmetricHeap
 
     M, N, K = 512, 384, 128
