@@ -265,3 +265,28 @@ def test_pack_matrix_moves_every_element_once(lib):
         want[:, :dcols] = 0
         want[:rows, :cols] = src.cpu()
         assert torch.equal(dst.cpu(), want), (dtype, rows, cols, sr, sc)
+
+
+def test_packed_operands_outlive_their_descriptor_only(lib):
+    """A packed operand belongs to the descriptor it was packed for: a second descriptor built while the first is
+    alive gets a buffer of its own (both launches then read what they were given), and the buffer is taken up again
+    once the descriptor that held it is gone."""
+    from tileccl_amd import _launch, _lib
+
+    M, N, K = 128, 128, 64
+    A1, A2 = seeded((K, M), 30).cuda().t(), seeded((K, M), 31).cuda().t()  # transposed views: packed
+    B = seeded((K, N), 32, scale=K**-0.5).cuda()
+    out1 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    out2 = torch.zeros_like(out1)
+    d1 = _launch.gemm_desc(A1, B, out1)
+    d2 = _launch.gemm_desc(A2, B, out2)
+    assert d1.A != d2.A and d1.A != A1.data_ptr() and d1.B == B.data_ptr()
+    for d in (d1, d2):
+        _lib.check(lib.tccl_gemm(C.byref(d), _launch.stream_ptr()), "tccl_gemm")
+    torch.cuda.synchronize()
+    assert_gemm_close(out1, A1.float().cpu() @ B.float().cpu(), tight=0.004)
+    assert_gemm_close(out2, A2.float().cpu() @ B.float().cpu(), tight=0.004)
+    first = d2.A
+    del d, d1, d2
+    d3 = _launch.gemm_desc(A1, B, out1)
+    assert d3.A == first  # the most recently released buffer of that shape
